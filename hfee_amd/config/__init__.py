@@ -4,5 +4,6 @@ from .specs import (NormSpec, PositionSpec, MixerSpec, FeedForwardSpec, LayerSpe
 from .llama import LlamaConfig, RopeScaling
 from .vofezen import VofezenConfig
 from .sabezen import SabezenConfig
+from .ronavik import RonavikConfig
 from .registry import (register_architecture, lookup_architecture, architecture_of,
                        architecture_names, config_from_dict, config_from_folder, model_spec_of)

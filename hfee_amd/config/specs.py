@@ -90,9 +90,13 @@ class LayerSpec:
     feed_forward_norm: NormSpec
     prefix: str          # tensor-name prefix of this layer, e.g. "model.layers.3."
     names: tuple = ()    # (role, tensor-name suffix) pairs overriding the parts' defaults
+    params: tuple = ()   # (name, value) pairs of the arrangement itself; see each block
 
     def name_of(self, role: str, default: str) -> str:
         return self.prefix + dict(self.names).get(role, default)
+
+    def get(self, name: str, default: Any = None):
+        return dict(self.params).get(name, default)
 
 
 @dataclass(frozen=True)

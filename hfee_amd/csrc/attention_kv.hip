@@ -14,6 +14,14 @@
 // softmax with a sink: the denominator holds one more term exp(sink_h), which has no key and
 // no value: p_j = exp(s_j - m) / (exp(sink_h - m) + sum_i exp(s_i - m)), m the maximum over
 // the scores and the sink.
+//
+// Without a softmax (`weighting` 1): a visible key weighs sigmoid(s_j + b_h), b_h a number a head (where
+// the softmax has its sinks); the weights are not normalized over the keys.
+//
+// qk_norm_write is the other way into the cache: no rotation; q and k are divided by their root mean
+// square over each head and multiplied by a weight shared by the heads, q also by a temperature that
+// grows with the logarithm of the position in steps of `every` tokens:
+// 1 + coef * ln(floor((p + 1) / every) + 1).
 #include "attention_kv.h"
 
 using namespace hfee;
@@ -80,6 +88,52 @@ __global__ __launch_bounds__(256) void kv_write_kernel(
   }
 }
 
+// ---------------------------------------------------------------- norm of q and k + cache write
+// One wave a (token, unit): the units of a token are its query heads (normed in place), its key heads
+// (normed into the token's slot) and its value heads (copied into the slot).  qw, kw: float32 [dk].
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_write_kernel(
+    T* __restrict__ q, int64_t ldq, int num_heads, const T* __restrict__ k, int64_t ldk, const T* __restrict__ v,
+    int64_t ldv, const float* __restrict__ qw, const float* __restrict__ kw, float eps, float temp_coef, int temp_every,
+    const int* __restrict__ positions, const int* __restrict__ token_segment, const int* __restrict__ block_tables,
+    int bt_stride, T* __restrict__ cache, KvLayout lay, int n) {
+  const int units = num_heads + (k != nullptr ? 2 * lay.kv_heads : 0);
+  const int64_t item = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (item >= (int64_t)n * units) return;
+  const int t = (int)(item / units), unit = (int)(item % units), lane = threadIdx.x & 63;
+  const int pos = positions[t];
+  if (unit < num_heads) {
+    T* p = q + (int64_t)t * ldq + (int64_t)unit * lay.dk;
+    float ss = 0.f;
+    for (int d = lane; d < lay.dk; d += 64) {
+      const float x = to_float<T>(p[d]);
+      ss = fmaf(x, x, ss);
+    }
+    float factor = 1.0f / sqrtf(wave_sum(ss) / (float)lay.dk + eps);
+    if (temp_every > 0) factor *= 1.0f + temp_coef * logf((float)((pos + 1) / temp_every) + 1.0f);
+    for (int d = lane; d < lay.dk; d += 64) p[d] = from_float<T>(to_float<T>(p[d]) * factor * qw[d]);
+    return;
+  }
+  const int page = block_tables[(int64_t)token_segment[t] * bt_stride + (pos >> lay.page_shift)];
+  const int slot = pos & (lay.page_size - 1);
+  if (unit < num_heads + lay.kv_heads) {
+    const int g = unit - num_heads;
+    const T* p = k + (int64_t)t * ldk + (int64_t)g * lay.dk;
+    float ss = 0.f;
+    for (int d = lane; d < lay.dk; d += 64) {
+      const float x = to_float<T>(p[d]);
+      ss = fmaf(x, x, ss);
+    }
+    const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)lay.dk + eps);
+    for (int d = lane; d < lay.dk; d += 64)
+      cache[lay.key_offset(page, g, slot, d)] = finite_for_cache<T>(from_float<T>(to_float<T>(p[d]) * inv * kw[d]));
+    return;
+  }
+  const int g = unit - num_heads - lay.kv_heads;
+  const T* p = v + (int64_t)t * ldv + (int64_t)g * lay.dv;
+  for (int d = lane; d < lay.dv; d += 64) cache[lay.value_offset(page, g, slot, d)] = finite_for_cache<T>(p[d]);
+}
+
 // ---------------------------------------------------------------- plain attention
 // Lane (j mod 64) owns key j, so which lane adds which term depends only on the key's
 // absolute position: a token's result does not change with the way the work was cut into
@@ -91,7 +145,7 @@ __global__ __launch_bounds__(64) void attention_kv_plain_kernel(
     T* __restrict__ out, int64_t ld_out, const T* __restrict__ q, int64_t ldq,
     const T* __restrict__ cache, KvLayout lay, const int* __restrict__ positions,
     const int* __restrict__ token_segment, const int* __restrict__ block_tables, int bt_stride,
-    int num_heads, float scale, const float* __restrict__ sinks) {
+    int num_heads, float scale, const float* __restrict__ sinks, int weighting) {
   extern __shared__ float lds[];
   const int dk = lay.dk, dv = lay.dv;
   float* qs = lds;            // [dk]
@@ -105,7 +159,7 @@ __global__ __launch_bounds__(64) void attention_kv_plain_kernel(
   __syncthreads();
 
   float m = -INFINITY;
-  for (int base = 0; base <= pos; base += 64) {
+  for (int base = 0; weighting == 0 && base <= pos; base += 64) {
     const int j = base + lane;
     if (j <= pos) {
       const T* kr = cache + lay.key_offset(bt[j >> lay.page_shift], kvh, j & (lay.page_size - 1), 0);
@@ -115,8 +169,8 @@ __global__ __launch_bounds__(64) void attention_kv_plain_kernel(
     }
   }
   m = wave_max(m);
-  const bool has_sink = sinks != nullptr;
-  const float sink = has_sink ? sinks[h] : 0.f;
+  const bool has_sink = sinks != nullptr && weighting == 0;
+  const float sink = sinks != nullptr ? sinks[h] : 0.f;      // (without a softmax: the number that joins every score)
   if (has_sink) m = fmaxf(m, sink);
 
   float lsum = 0.f;
@@ -130,7 +184,7 @@ __global__ __launch_bounds__(64) void attention_kv_plain_kernel(
       const T* kr = cache + lay.key_offset(bt[j >> lay.page_shift], kvh, j & (lay.page_size - 1), 0);
       float s = 0.f;
       for (int d = 0; d < dk; ++d) s = fmaf(qs[d], to_float<T>(kr[d]), s);
-      e = expf(s * scale - m);
+      e = weighting == 0 ? expf(s * scale - m) : 1.0f / (1.0f + expf(-(s * scale + sink)));
       lsum += e;
     }
     __syncthreads();
@@ -149,6 +203,7 @@ __global__ __launch_bounds__(64) void attention_kv_plain_kernel(
   }
   lsum = wave_sum(lsum);
   if (has_sink) lsum += expf(sink - m);
+  if (weighting != 0) lsum = 1.0f;
 #pragma unroll
   for (int r = 0; r < kMaxDvPerLane; ++r) {
     const int d = lane + 64 * r;
@@ -260,12 +315,42 @@ HFEE_API int hfee_kv_write(void* q, int64_t ldq, int num_heads, int q_dim, int q
   return 0;
 }
 
+HFEE_API int hfee_qk_norm_write(void* q, int64_t ldq, int num_heads, const void* k, int64_t ldk, const void* v, int64_t ldv,
+                                int dtype, const float* q_weight, const float* k_weight, float eps, float temp_coef,
+                                int temp_every, const int* positions, const int* token_segment, const int* block_tables,
+                                int bt_stride, void* cache, int kv_heads, int dk, int dv, int page_size, int n,
+                                hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && num_heads > 0 && q != nullptr && q_weight != nullptr && eps >= 0.f, "qk_norm_write: bad arguments");
+  if (n == 0) return 0;
+  KvLayout lay;
+  if (make_kv_layout(&lay, kv_heads, dk, dv, page_size)) return 1;
+  HFEE_REQUIRE(ldq >= (int64_t)num_heads * dk, "qk_norm_write: q rows too short");
+  if (k != nullptr) {
+    HFEE_REQUIRE(v != nullptr && cache != nullptr && k_weight != nullptr && token_segment != nullptr && block_tables != nullptr,
+                 "qk_norm_write: k, v, the keys' weight, the cache and the block tables come together");
+    HFEE_REQUIRE(ldk >= (int64_t)kv_heads * dk && ldv >= (int64_t)kv_heads * dv, "qk_norm_write: k/v rows too short");
+  }
+  const int64_t items = (int64_t)n * (num_heads + (k != nullptr ? 2 * kv_heads : 0));
+  HFEE_REQUIRE((items + 3) / 4 <= 0x7fffffff, "qk_norm_write: too much work for one launch");
+#define LAUNCH(T)                                                                                                    \
+  qk_norm_write_kernel<T><<<(unsigned)((items + 3) / 4), 256, 0, stream>>>((T*)q, ldq, num_heads, (const T*)k, ldk,  \
+      (const T*)v, ldv, q_weight, k_weight, eps, temp_coef, temp_every, positions, token_segment, block_tables,      \
+      bt_stride, (T*)cache, lay, n)
+  if (dtype == 0) LAUNCH(float);
+  else if (dtype == 1) LAUNCH(bf16_t);
+  else return fail("qk_norm_write: unknown dtype %d", dtype);
+#undef LAUNCH
+  HFEE_CHECK_LAUNCH("qk_norm_write");
+  return 0;
+}
+
 HFEE_API int hfee_attention_kv_plain(void* out, int64_t ld_out, const void* q, int64_t ldq, const void* cache,
                                      int dtype, const int* positions, const int* token_segment,
                                      const int* block_tables, int bt_stride, int num_heads, int kv_heads, int dk,
-                                     int dv, int page_size, float scale, const float* sinks, int n,
+                                     int dv, int page_size, float scale, const float* sinks, int weighting, int n,
                                      hipStream_t stream) {
   HFEE_REQUIRE(n >= 0, "attention_kv_plain: bad token count");
+  HFEE_REQUIRE(weighting == 0 || weighting == 1, "attention_kv_plain: the weights are a softmax's (0) or sigmoids (1)");
   if (n == 0) return 0;
   HFEE_REQUIRE(num_heads > 0 && kv_heads > 0 && num_heads % kv_heads == 0,
                "attention_kv_plain: %d heads are not a multiple of %d kv heads", num_heads, kv_heads);
@@ -279,10 +364,10 @@ HFEE_API int hfee_attention_kv_plain(void* out, int64_t ld_out, const void* q, i
   const size_t lds = (dk + 64) * sizeof(float);
   if (dtype == 0)
     attention_kv_plain_kernel<float><<<grid, 64, lds, stream>>>((float*)out, ld_out, (const float*)q, ldq,
-        (const float*)cache, lay, positions, token_segment, block_tables, bt_stride, num_heads, scale, sinks);
+        (const float*)cache, lay, positions, token_segment, block_tables, bt_stride, num_heads, scale, sinks, weighting);
   else if (dtype == 1)
     attention_kv_plain_kernel<bf16_t><<<grid, 64, lds, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq,
-        (const bf16_t*)cache, lay, positions, token_segment, block_tables, bt_stride, num_heads, scale, sinks);
+        (const bf16_t*)cache, lay, positions, token_segment, block_tables, bt_stride, num_heads, scale, sinks, weighting);
   else
     return fail("attention_kv_plain: unknown dtype %d", dtype);
   HFEE_CHECK_LAUNCH("attention_kv_plain");

@@ -15,6 +15,10 @@
 //   1  a single token: up to 16 query heads that share a key/value head; the keys may be
 //      split over several waves, whose partial results a second kernel joins.
 // The sink joins the denominator once, at the very end.
+//
+// Compiled with -DHFEE_KV_WEIGHTS=1 there is no softmax: a visible key weighs sigmoid(score + b_h), b_h a
+// number a head (given where the softmax has its sinks), nothing is normalized over the keys, and the
+// splits of a single token's keys are plain sums.
 #include "attention_kv.h"
 
 #ifndef HFEE_DK
@@ -25,7 +29,11 @@ using namespace hfee;
 
 namespace {
 
+#ifndef HFEE_KV_WEIGHTS
+#define HFEE_KV_WEIGHTS 0
+#endif
 constexpr int DK = HFEE_DK, DV = HFEE_DV;
+constexpr bool SIGMOID = HFEE_KV_WEIGHTS == 1;
 static_assert(DK % 16 == 0 && DV % 16 == 0 && DK >= 16 && DV >= 16, "key and value sizes are multiples of 16");
 constexpr int KSTEPS = (DK + 31) / 32;     // steps of 32 dims (the last may be half empty)
 constexpr int VBLOCKS = DV / 16;
@@ -54,6 +62,18 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
 // has any (the same answer in every lane).
 __device__ __forceinline__ void weigh_tile(f32x4 (&s)[2], float& reference, float& lsum, f32x4 (&acc)[VBLOCKS],
                                            Operand& pop, int j0, int g, int pos, float scale_log2, bool masked) {
+  if constexpr (SIGMOID) {      // `reference` is the head's number (in base 2), and stays
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = 1.0f / (1.0f + __builtin_amdgcn_exp2f(-fmaf(s[kb][i], scale_log2, reference)));
+        s[kb][i] = masked && j0 + kb * 16 + g * 4 + i > pos ? 0.f : p;
+      }
+    pop.u = u32x4{pack_bf16(s[0][0], s[0][1]), pack_bf16(s[0][2], s[0][3]), pack_bf16(s[1][0], s[1][1]),
+                  pack_bf16(s[1][2], s[1][3])};
+    return;
+  }
   float tmax = -INFINITY;
 #pragma unroll
   for (int kb = 0; kb < 2; ++kb)
@@ -166,7 +186,7 @@ __global__ __launch_bounds__(256) void attention_kv_kernel(
   float m[RB], lsum[RB];
 #pragma unroll
   for (int b = 0; b < RB; ++b) {
-    m[b] = -INFINITY; lsum[b] = 0.f;
+    m[b] = SIGMOID ? (sinks != nullptr ? sinks[head[b]] * kLog2e : 0.f) : -INFINITY; lsum[b] = 0.f;
 #pragma unroll
     for (int vb = 0; vb < VBLOCKS; ++vb) acc[b][vb] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
@@ -285,7 +305,8 @@ __global__ __launch_bounds__(256) void attention_kv_kernel(
     l += __shfl_xor(l, 32, 64);
     if (splits == 1) {
       float a = 1.f;
-      if (sinks != nullptr) {
+      if constexpr (SIGMOID) l = 1.f;
+      if (!SIGMOID && sinks != nullptr) {
         const float sk = sinks[head[b]] * kLog2e;
         const float m_all = fmaxf(m[b], sk);
         a = exp2f(m[b] - m_all);
@@ -370,7 +391,7 @@ __global__ __launch_bounds__(256) void attention_kv_shared_kernel(
   float m[RB], lsum[RB];
 #pragma unroll
   for (int b = 0; b < RB; ++b) {
-    m[b] = -INFINITY; lsum[b] = 0.f;
+    m[b] = SIGMOID ? (sinks != nullptr ? sinks[head] * kLog2e : 0.f) : -INFINITY; lsum[b] = 0.f;
 #pragma unroll
     for (int vb = 0; vb < VBLOCKS; ++vb) acc[b][vb] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
@@ -496,7 +517,8 @@ __global__ __launch_bounds__(256) void attention_kv_shared_kernel(
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
     float a = 1.f;
-    if (sinks != nullptr) {
+    if constexpr (SIGMOID) l = 1.f;
+    if (!SIGMOID && sinks != nullptr) {
       const float sk = sinks[head] * kLog2e;
       const float m_all = fmaxf(m[b], sk);
       a = exp2f(m[b] - m_all);
@@ -523,13 +545,14 @@ __global__ __launch_bounds__(64) void attention_kv_join_kernel(
   const int item = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const float* pr = partial + ((int64_t)item * num_heads + head) * splits * kPartial;
   const int token = items[item * 4];
-  const float sk = sinks != nullptr ? sinks[head] * kLog2e : -INFINITY;
+  const float sk = !SIGMOID && sinks != nullptr ? sinks[head] * kLog2e : -INFINITY;
   const float my_m = lane < splits ? pr[lane * kPartial] : -INFINITY;
   const float my_l = lane < splits ? pr[lane * kPartial + 1] : 0.f;
   const float m = fmaxf(wave_max(my_m), sk);
-  const float my_w = exp2f(my_m - m);               // (0 for a split without keys and for lanes beyond the splits)
-  const float lsum = wave_sum(my_l * my_w) + (sinks != nullptr ? exp2f(sk - m) : 0.f);
-  const float inv = 1.0f / lsum;
+  // (0 for a split without keys and for lanes beyond the splits; without a softmax every split counts as it is)
+  const float my_w = SIGMOID ? (lane < splits ? 1.f : 0.f) : exp2f(my_m - m);
+  const float lsum = wave_sum(my_l * my_w) + (!SIGMOID && sinks != nullptr ? exp2f(sk - m) : 0.f);
+  const float inv = SIGMOID ? 1.0f : 1.0f / lsum;
   for (int d = lane; d < DV; d += 64) {
     float o = 0.f;
 #pragma unroll 8
@@ -544,6 +567,7 @@ HFEE_DEFINE_LAST_ERROR
 
 HFEE_API int hfee_attention_kv_bf16_dk() { return DK; }
 HFEE_API int hfee_attention_kv_bf16_dv() { return DV; }
+HFEE_API int hfee_attention_kv_bf16_weights() { return HFEE_KV_WEIGHTS; }
 // the most rows of an item of mode 0, for this many query heads a key/value head (where they are a
 // multiple of four, the kernel that shares the key tiles through LDS runs)
 HFEE_API int hfee_attention_kv_bf16_rows(int heads_per_kv_head) {

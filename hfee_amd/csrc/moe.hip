@@ -7,6 +7,13 @@
 //   up:    act[t][j][f] = silu(W_gate[e][f] . h_t) * (W_up[e][f] . h_t),   e = the j-th expert of t
 //   down:  x[t][c] (+)= sum_j weight_tj (W_down[e_j][c] . act[t][j])
 //
+// Experts without a gate (`form` 1, no W_gate): act[t][j][f] = relu(w_tj (W_up[e][f] . h_t))^2, where w_tj
+// (in_weights, or one) multiplies the expert's input: a product is linear, so the number meets the sum in
+// float32 before the activation instead of every element of h before it is rounded.
+//
+// router_topk: scores sigmoid(z) of router logits z (float32 [n, experts]); the `top` largest choose a
+// token's experts (the lower number of two equal ones), its pair weights are the chosen scores as they are.
+//
 // The experts' matrices are stacked [experts][rows][columns].  Two forms:
 //
 // Token by token (moe_up, moe_down): a wave a dot product, lanes over the summed dimension, added up in a
@@ -74,21 +81,28 @@ __global__ __launch_bounds__(256) void moe_up_kernel(T* __restrict__ act, const 
                                                      const T* __restrict__ w_gate, const T* __restrict__ w_up,
                                                      const int* __restrict__ chosen, const int* __restrict__ table,
                                                      const int* __restrict__ token_ids, int top, int experts, int F,
-                                                     int width) {
+                                                     int width, const float* __restrict__ in_weights) {
   const int pair = blockIdx.x, t = pair / top, j = pair - t * top;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int e = expert_of(chosen, table, token_ids, t, j, top);
   if (e < 0 || e >= experts) return;                       // (a table that names no such expert: nothing is read)
   const T* hr = h + (int64_t)t * ldh;
-  const bool wide = rows_aligned<T>(w_gate, h, width, ldh) && (uintptr_t)w_up % 16 == 0;
+  const bool wide = rows_aligned<T>(w_up, h, width, ldh) && (uintptr_t)w_gate % 16 == 0;
   const int f0 = (blockIdx.y * 4 + wave) * kRowsPerWave;
+  const float wt = in_weights != nullptr ? in_weights[pair] : 1.0f;
 #pragma unroll
   for (int r = 0; r < kRowsPerWave; ++r) {
     const int f = f0 + r;
     if (f >= F) break;
-    const T* g = w_gate + ((int64_t)e * F + f) * width;
     const T* u = w_up + ((int64_t)e * F + f) * width;
     float sg, su;
+    if (w_gate == nullptr) {        // no gate: the square of relu
+      two_dots<T>(u, nullptr, hr, width, lane, wide, su, sg);
+      su = fmaxf(wave_sum(su) * wt, 0.f);
+      if (lane == 0) act[(int64_t)pair * F + f] = from_float<T>(su * su);
+      continue;
+    }
+    const T* g = w_gate + ((int64_t)e * F + f) * width;
     two_dots<T>(g, u, hr, width, lane, wide, sg, su);
     sg = wave_sum(sg);
     su = wave_sum(su);
@@ -214,10 +228,12 @@ __device__ __forceinline__ void tile_products(f32x4 (&acc)[NB][4][4], const bf16
   }
 }
 
+template <int FORM>
 __global__ __launch_bounds__(256) void moe_group_up_kernel(bf16_t* __restrict__ act, const bf16_t* __restrict__ h, int64_t ldh,
                                                            const bf16_t* __restrict__ w_gate, const bf16_t* __restrict__ w_up,
                                                            const int* __restrict__ order, const int* __restrict__ tiles,
-                                                           int most_tiles, int top, int F, int width) {
+                                                           int most_tiles, int top, int F, int width,
+                                                           const float* __restrict__ in_weights) {
   if ((int)blockIdx.x >= tiles[3 * most_tiles]) return;
   const int* tl = tiles + 3 * blockIdx.x;
   const int e = tl[0], first = tl[1], count = tl[2];
@@ -231,6 +247,26 @@ __global__ __launch_bounds__(256) void moe_group_up_kernel(bf16_t* __restrict__ 
     const int r = mt * 16 + r16;
     pair[mt] = order[first + (r < count ? r : 0)];
     a_rows[mt] = h + (int64_t)(pair[mt] / top) * ldh;
+  }
+  if constexpr (FORM == 1) {      // no gate: the square of relu, the pair's weight on the sum
+    const bf16_t* const b1[1] = {w_up + (int64_t)e * F * width};
+    f32x4 acc1[1][4][4] = {};
+    tile_products<1>(acc1, a_rows, b1, width, row0, F, lane);
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+      if (mt * 16 + r16 >= count) continue;
+      const float wt = in_weights != nullptr ? in_weights[pair[mt]] : 1.0f;
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) {
+        const int f = row0 + nt * 16 + (lane >> 4) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float u = fmaxf(acc1[0][nt][mt][i] * wt, 0.f);
+          if (f + i < F) act[(int64_t)pair[mt] * F + f + i] = float_to_bf16(u * u);
+        }
+      }
+    }
+    return;
   }
   const bf16_t* const b[2] = {w_gate + (int64_t)e * F * width, w_up + (int64_t)e * F * width};
   f32x4 acc[2][4][4] = {};
@@ -302,7 +338,50 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x,
   }
 }
 
+// One wave a token.  A lane looks through its share of the experts (lane, lane + 64, ...) for the largest
+// logit that is not chosen yet (a bit a share in the lane's own registers says which are); the wave's lanes
+// meet over (logit, number), the larger logit and of two equal ones the lower number, and every lane ends
+// with the same answer.  The sigmoid grows with its argument, so the largest scores are the largest logits.
+constexpr int kRouterMostExperts = 64 * 128;
+
+__global__ __launch_bounds__(256) void router_topk_kernel(const float* __restrict__ logits, int64_t ld, int n, int experts,
+                                                          int top, int* __restrict__ chosen, float* __restrict__ weights) {
+  const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (t >= n) return;
+  const float* z = logits + (int64_t)t * ld;
+  unsigned long long taken[2] = {0ull, 0ull};
+  for (int j = 0; j < top; ++j) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+    for (int e = lane, i = 0; e < experts; e += 64, ++i) {
+      const float v = z[e];
+      if (!((taken[i >> 6] >> (i & 63)) & 1ull) && (at == 0x7fffffff || v > best)) { best = v; at = e; }
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+      const float ob = __shfl_xor(best, off, 64);
+      const int oa = __shfl_xor(at, off, 64);
+      if (oa != 0x7fffffff && (at == 0x7fffffff || ob > best || (ob == best && oa < at))) { best = ob; at = oa; }
+    }
+    if ((at & 63) == lane) taken[(at >> 6) >> 6] |= 1ull << ((at >> 6) & 63);
+    if (lane == 0) {
+      chosen[(int64_t)t * top + j] = at;
+      weights[(int64_t)t * top + j] = 1.0f / (1.0f + expf(-best));
+    }
+  }
+}
+
 }  // namespace
+
+HFEE_API int hfee_router_topk(const float* logits, int64_t ld, int n, int experts, int top, int* chosen, float* weights,
+                              hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && experts >= 1 && experts <= kRouterMostExperts && top >= 1 && top <= experts && ld >= experts,
+               "router_topk: a token uses 1 to %d experts (of at most %d), not %d", experts, kRouterMostExperts, top);
+  if (n == 0) return 0;
+  router_topk_kernel<<<(n + 3) / 4, 256, 0, stream>>>(logits, ld, n, experts, top, chosen, weights);
+  HFEE_CHECK_LAUNCH("router_topk");
+  return 0;
+}
 
 // The whole feed-forward in its grouped form, bfloat16: x (float32 [n, width]) += the experts' weighted
 // outputs.  order: int32 [n * top]; tiles: int32 [3 * hfee_moe_group_tiles(n, top, experts) + 1]; act:
@@ -314,11 +393,12 @@ HFEE_API int hfee_moe_group_tiles(int n, int top, int experts) {
 HFEE_API int hfee_moe_grouped(float* x, int64_t ldx, const void* h, int64_t ldh, const void* w_gate, const void* w_up,
                               const void* w_down, const int* chosen, const int* table, const int* token_ids,
                               const float* pair_weights, float weight, int top, int experts, int ff, int width, int n,
-                              int* order, int* tiles, void* act, float* y, hipStream_t stream) {
+                              int* order, int* tiles, void* act, float* y, const float* in_weights, hipStream_t stream) {
   HFEE_REQUIRE(n >= 0 && top >= 1 && experts >= 1 && experts <= 8192 && ff >= 1 && width >= 1, "moe_grouped: bad sizes");
   HFEE_REQUIRE(chosen != nullptr || (table != nullptr && token_ids != nullptr), "moe_grouped: the experts of a token, or a table and the ids");
   HFEE_REQUIRE(width % 32 == 0 && ff % 32 == 0 && ldh % 8 == 0 && ldx >= width && ldh >= width,
                "moe_grouped: the width and the experts' size must be multiples of 32");
+  HFEE_REQUIRE(w_gate != nullptr || pair_weights == nullptr, "moe_grouped: experts without a gate take their weights on the input");
   HFEE_REQUIRE(((uintptr_t)h | (uintptr_t)w_gate | (uintptr_t)w_up | (uintptr_t)w_down | (uintptr_t)act) % 16 == 0,
                "moe_grouped: operands must be 16-byte aligned");
   HFEE_REQUIRE(order != nullptr && tiles != nullptr && act != nullptr && (top == 1 || y != nullptr), "moe_grouped: scratch missing");
@@ -327,8 +407,12 @@ HFEE_API int hfee_moe_grouped(float* x, int64_t ldx, const void* h, int64_t ldh,
   const int most = hfee_moe_group_tiles(n, top, experts);
   moe_group_kernel<<<1, 1024, 4 * experts * sizeof(int), stream>>>(order, tiles, most, chosen, table, token_ids, n, top, experts);
   HFEE_CHECK_LAUNCH("moe_group");
-  moe_group_up_kernel<<<dim3(most, (ff + kTileRows - 1) / kTileRows), 256, 0, stream>>>(
-      (bf16_t*)act, (const bf16_t*)h, ldh, (const bf16_t*)w_gate, (const bf16_t*)w_up, order, tiles, most, top, ff, width);
+  if (w_gate != nullptr)
+    moe_group_up_kernel<0><<<dim3(most, (ff + kTileRows - 1) / kTileRows), 256, 0, stream>>>(
+        (bf16_t*)act, (const bf16_t*)h, ldh, (const bf16_t*)w_gate, (const bf16_t*)w_up, order, tiles, most, top, ff, width, nullptr);
+  else
+    moe_group_up_kernel<1><<<dim3(most, (ff + kTileRows - 1) / kTileRows), 256, 0, stream>>>(
+        (bf16_t*)act, (const bf16_t*)h, ldh, nullptr, (const bf16_t*)w_up, order, tiles, most, top, ff, width, in_weights);
   HFEE_CHECK_LAUNCH("moe_group_up");
   moe_group_down_kernel<<<dim3(most, (width + kTileRows - 1) / kTileRows), 256, 0, stream>>>(
       top == 1 ? x : y, top == 1 ? ldx : (int64_t)width, (const bf16_t*)act, (const bf16_t*)w_down, order, tiles, most, ff, width,
@@ -345,7 +429,7 @@ HFEE_API int hfee_moe_grouped(float* x, int64_t ldx, const void* h, int64_t ldh,
 
 HFEE_API int hfee_moe_up(void* act, const void* h, int64_t ldh, const void* w_gate, const void* w_up, int dtype,
                          const int* chosen, const int* table, const int* token_ids, int top, int experts, int ff,
-                         int width, int n, hipStream_t stream) {
+                         int width, int n, const float* in_weights, hipStream_t stream) {
   HFEE_REQUIRE(n >= 0 && top >= 1 && experts >= 1 && ff >= 1 && width >= 1 && ldh >= width, "moe_up: bad sizes");
   HFEE_REQUIRE(chosen != nullptr || (table != nullptr && token_ids != nullptr), "moe_up: the experts of a token, or a table and the ids");
   if (n == 0) return 0;
@@ -354,10 +438,10 @@ HFEE_API int hfee_moe_up(void* act, const void* h, int64_t ldh, const void* w_ga
   dim3 grid((unsigned)((int64_t)n * top), (ff + per_block - 1) / per_block);
   if (dtype == 0)
     moe_up_kernel<float><<<grid, 256, 0, stream>>>((float*)act, (const float*)h, ldh, (const float*)w_gate, (const float*)w_up,
-                                                   chosen, table, token_ids, top, experts, ff, width);
+                                                   chosen, table, token_ids, top, experts, ff, width, in_weights);
   else if (dtype == 1)
     moe_up_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)act, (const bf16_t*)h, ldh, (const bf16_t*)w_gate,
-                                                    (const bf16_t*)w_up, chosen, table, token_ids, top, experts, ff, width);
+                                                    (const bf16_t*)w_up, chosen, table, token_ids, top, experts, ff, width, in_weights);
   else
     return fail("moe_up: unknown dtype %d", dtype);
   HFEE_CHECK_LAUNCH("moe_up");

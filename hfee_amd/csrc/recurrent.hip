@@ -6,6 +6,8 @@
 //   rule 0 (gated linear attention):  S <- diag(a_t) S + k_t v_t^T;                    o_t = S^T q_t
 //   rule 1 (gated delta rule):        S <- diag(a_t) S;  u = b_t (v_t - S^T k_t);
 //                                     S <- S + k_t u^T;                                o_t = S^T q_t
+//   rule 2 (state-space duality):     S <- diag(a_t) S + k_t (b_t v_t)^T;              o_t = S^T q_t
+//                                     (b_t the step size a head; with `decay_per_head` a_t is one number a head)
 //
 // `linear_scan` walks the tokens that a step brings for a request one after the other, from the
 // state that the steps before left in the request's slot, and leaves the new state there: a
@@ -15,15 +17,20 @@
 // head lies in blocks of four columns, each in the order in which a wave's lanes hold it.
 //
 // Around it, each in float32 whatever the engine's dtype:
-//   short_conv_silu     y_t = silu(sum_j taps[K-1-j] x_(t-j)) per channel, the K-1 inputs before the
-//                       step's first token from the slot's state (zeros at a sequence's start)
-//   short_conv_keep     the slot's state <- the last K-1 inputs
+//   short_conv          y_t = act(sum_j taps[K-1-j] (x_(t-j) + in_bias) + out_bias) per channel, act the SiLU or
+//                       nothing, the K-1 inputs before the step's first token from the slot's state (zeros at a
+//                       sequence's start, also where the inputs have a bias)
+//   short_conv_keep     the slot's state <- the last K-1 inputs (with their bias)
 //   unit_heads          x / sqrt(sum(x^2) + eps) * factor over each head
 //   scan_gate           what a projection becomes before it enters the recurrence:
 //                       0  exp(-exp(A[head]) softplus(z + bias))      (a decay from a step size)
 //                       1  exp(logsigmoid(z + bias) / tau)            (a decay sigmoid(z)^(1/tau))
 //                       2  sigmoid(z)                                 (a writing strength)
 //                       3  z * factor for the first columns, z for the rest (a cast)
+//                       4  softplus(z + bias)                         (a step size)
+//   rglru_scan          the real-gated linear recurrent unit, a number a channel:
+//                       a = exp(rate * sigmoid(r)), S <- a S + sqrt(1 - a^2) sigmoid(i) u, out = S * gelu(y + bias)
+//   gate_group_norm     out = norm((o + D[head] x) * silu(z)) * weight, the norm over each of `groups` equal parts
 //   head_norm_gate      out = o / sqrt(mean(o^2) + eps) * weight * act(gate) over each head,
 //                       act the sigmoid or the SiLU, in the engine's dtype for the product behind it
 #include "common.h"
@@ -37,11 +44,20 @@ __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - l
 
 // x: [n, C] rows of the step; state: [slots][K-1][C], index K-2 the newest; taps: float32 [C][K], the
 // last column the current token's; y: float32 [n, C].
+// An input's bias is added before the input is rounded to T, in the step's rows here as in the rows
+// that short_conv_keep leaves in the state: a token's result does not depend on where its sequence was cut.
+template <typename T>
+__device__ __forceinline__ float conv_input(const T* p, const float* in_bias, int c) {
+  const float v = to_float<T>(*p);
+  return in_bias != nullptr ? to_float<T>(from_float<T>(v + in_bias[c])) : v;
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void short_conv_silu_kernel(
     float* __restrict__ y, int64_t ldy, const T* __restrict__ x, int64_t ldx, const T* __restrict__ state,
     const float* __restrict__ taps, const int* __restrict__ token_segment, const int* __restrict__ segment_rows,
-    const int* __restrict__ segment_slots, int C, int K) {
+    const int* __restrict__ segment_slots, int C, int K, const float* __restrict__ in_bias,
+    const float* __restrict__ out_bias, int act) {
   const int t = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= C) return;
   const int seg = token_segment[t];
@@ -50,23 +66,26 @@ __global__ __launch_bounds__(256) void short_conv_silu_kernel(
   float sum = 0.f;
   for (int j = K - 1; j >= 0; --j) {                        // the oldest input first
     const int at = i - j;
-    const float v = at >= 0 ? to_float<T>(x[(int64_t)(t - j) * ldx + c]) : to_float<T>(st[(int64_t)(K - 1 + at) * C + c]);
+    const float v = at >= 0 ? conv_input<T>(x + (int64_t)(t - j) * ldx + c, in_bias, c) : to_float<T>(st[(int64_t)(K - 1 + at) * C + c]);
     sum = fmaf(taps[(int64_t)c * K + (K - 1 - j)], v, sum);
   }
-  y[(int64_t)t * ldy + c] = sum / (1.0f + expf(-sum));
+  if (out_bias != nullptr) sum += out_bias[c];
+  y[(int64_t)t * ldy + c] = act == 1 ? sum / (1.0f + expf(-sum)) : sum;
 }
 
 template <typename T>
 __global__ __launch_bounds__(256) void short_conv_keep_kernel(
     T* __restrict__ state, const T* __restrict__ x, int64_t ldx, const int* __restrict__ segment_rows,
-    const int* __restrict__ segment_lengths, const int* __restrict__ segment_slots, int C, int K) {
+    const int* __restrict__ segment_lengths, const int* __restrict__ segment_slots, int C, int K,
+    const float* __restrict__ in_bias) {
   const int seg = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= C) return;
   const int len = segment_lengths[seg], row0 = segment_rows[seg];
   T* st = state + (int64_t)segment_slots[seg] * (K - 1) * C;
   for (int m = 0; m < K - 1; ++m) {                         // ascending: what is read lies behind what was written
     const int i = len - (K - 1) + m;
-    st[(int64_t)m * C + c] = i >= 0 ? x[(int64_t)(row0 + i) * ldx + c] : st[(int64_t)(m + len) * C + c];
+    st[(int64_t)m * C + c] = i >= 0 ? from_float<T>(conv_input<T>(x + (int64_t)(row0 + i) * ldx + c, in_bias, c))
+                                    : st[(int64_t)(m + len) * C + c];
   }
 }
 
@@ -97,6 +116,7 @@ __global__ __launch_bounds__(256) void scan_gate_kernel(float* __restrict__ out,
   if (mode == 0) r = expf(-expf(per_head[c / head_width]) * softplus(v));
   else if (mode == 1) r = expf(log_sigmoid(v) / number);
   else if (mode == 2) r = 1.0f / (1.0f + expf(-v));
+  else if (mode == 4) r = softplus(v);
   else r = c < first_columns ? v * number : v;
   out[t * ldo + c] = r;
 }
@@ -177,7 +197,8 @@ __global__ __launch_bounds__(kScanWaves * 64) void linear_scan_kernel(
     float* __restrict__ out, int64_t ldo, float* __restrict__ state, const float* __restrict__ q, int64_t ldq,
     const float* __restrict__ k, int64_t ldk, const float* __restrict__ v, int64_t ldv, const float* __restrict__ decay,
     int64_t ldd, const float* __restrict__ beta, int64_t ldb, const int* __restrict__ segment_rows,
-    const int* __restrict__ segment_lengths, const int* __restrict__ segment_slots, int heads, int qk_heads, int D, int V) {
+    const int* __restrict__ segment_lengths, const int* __restrict__ segment_slots, int heads, int qk_heads, int D, int V,
+    int decay_per_head) {
   typedef ScanShape<DPT> Sh;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int seg = blockIdx.z, h = blockIdx.y, tid = threadIdx.x;
@@ -203,8 +224,9 @@ __global__ __launch_bounds__(kScanWaves * 64) void linear_scan_kernel(
     float kk[DPT], qq[DPT], aa[DPT];
     const float* kp = k + row * ldk + (int64_t)g * D + d0;
     const float* qp = q + row * ldq + (int64_t)g * D + d0;
-    const float* ap = decay + row * ldd + (int64_t)h * D + d0;
-    if (DPT % 4 == 0 && D == DPT * kScanParts && (((uintptr_t)kp | (uintptr_t)qp | (uintptr_t)ap) & 15) == 0) {
+    const float* ap = decay + row * ldd + (decay_per_head ? (int64_t)h : (int64_t)h * D + d0);
+    const int astep = decay_per_head ? 0 : 1;
+    if (!decay_per_head && DPT % 4 == 0 && D == DPT * kScanParts && (((uintptr_t)kp | (uintptr_t)qp | (uintptr_t)ap) & 15) == 0) {
       typedef float f32x4_t __attribute__((ext_vector_type(4)));      // (sixteen bytes a load where the rows allow)
 #pragma unroll
       for (int i = 0; i + 3 < DPT; i += 4) {
@@ -223,7 +245,7 @@ __global__ __launch_bounds__(kScanWaves * 64) void linear_scan_kernel(
         const bool in = d0 + i < D;
         kk[i] = in ? kp[i] : 0.f;
         qq[i] = in ? qp[i] : 0.f;
-        aa[i] = in ? ap[i] : 0.f;
+        aa[i] = in ? ap[i * astep] : 0.f;
       }
     }
     if constexpr (RULE == 1) {
@@ -235,6 +257,7 @@ __global__ __launch_bounds__(kScanWaves * 64) void linear_scan_kernel(
       }
       u = beta[row * ldb + h] * (u - column_sum(p0 + p1));
     }
+    if constexpr (RULE == 2) u *= beta[row * ldb + h];
     float o0 = 0.f, o1 = 0.f;
 #pragma unroll
     for (int i = 0; i < DPT; ++i) {
@@ -259,7 +282,7 @@ __global__ __launch_bounds__(kScanWaves * 64) void linear_scan_kernel(
       if (first + t < len && d < D) {
         const int64_t row = row0 + first + t;
         x = which == 0 ? k[row * ldk + (int64_t)g * D + d] : which == 1 ? q[row * ldq + (int64_t)g * D + d]
-                                                                      : decay[row * ldd + (int64_t)h * D + d];
+                                                                      : decay[row * ldd + (decay_per_head ? (int64_t)h : (int64_t)h * D + d)];
       }
       wide[r] = x;
     }
@@ -268,13 +291,13 @@ __global__ __launch_bounds__(kScanWaves * 64) void linear_scan_kernel(
       const int column = blockIdx.x * kScanWaves * kScanColumns + cc;
       narrow = t < Sh::TB && first + t < len && column < V ? v[(int64_t)(row0 + first + t) * ldv + (int64_t)h * V + column] : 0.f;
     }
-    if (RULE == 1 && tid < Sh::TB) strength = first + tid < len ? beta[(int64_t)(row0 + first + tid) * ldb + h] : 0.f;
+    if (RULE != 0 && tid < Sh::TB) strength = first + tid < len ? beta[(int64_t)(row0 + first + tid) * ldb + h] : 0.f;
   };
   auto put = [&](float* buffer) {
 #pragma unroll
     for (int r = 0; r < Sh::PER_THREAD; ++r) buffer[tid + r * kScanWaves * 64] = wide[r];
     if (tid < Sh::TB * kScanWaves * kScanColumns) buffer[Sh::WIDE + tid] = narrow;
-    if (RULE == 1 && tid < Sh::TB) buffer[Sh::WIDE + Sh::TB * kScanWaves * kScanColumns + tid] = strength;
+    if (RULE != 0 && tid < Sh::TB) buffer[Sh::WIDE + Sh::TB * kScanWaves * kScanColumns + tid] = strength;
   };
 
   ask(0);
@@ -299,6 +322,7 @@ __global__ __launch_bounds__(kScanWaves * 64) void linear_scan_kernel(
         }
         u = now.b * (now.v - column_sum(p0 + p1));
       }
+      if constexpr (RULE == 2) u = now.b * now.v;
       float o0 = 0.f, o1 = 0.f;
 #pragma unroll
       for (int i = 0; i < DPT; ++i) {
@@ -340,21 +364,100 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(T* __restrict__ out
   }
 }
 
+// The real-gated linear recurrent unit: one number a channel and request.  A thread owns a channel and
+// walks the tokens that the step brings for a request in order; what a token needs (its two gates, its
+// input, the other branch) is asked for kRgTokens tokens at a time, all at once, and the chain from token
+// to token is one multiply-add.  gates: float32 [n][blocks][2 * block] before their biases and sigmoids,
+// a block's decay gates, then its input gates.  rate: float32 [W], what the decay gate is multiplied by
+// to give the decay's logarithm (not positive).
+constexpr int kRgTokens = 8;
+
+template <typename T>
+__global__ __launch_bounds__(256) void rglru_scan_kernel(
+    T* __restrict__ out, int64_t ldo, float* __restrict__ state, const float* __restrict__ gates, int64_t ldg,
+    const float* __restrict__ gate_bias, const float* __restrict__ u, int64_t ldu, const float* __restrict__ rate,
+    const T* __restrict__ y, int64_t ldy, const float* __restrict__ y_bias, const int* __restrict__ segment_rows,
+    const int* __restrict__ segment_lengths, const int* __restrict__ segment_slots, int W, int block) {
+  const int seg = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= W) return;
+  const int b = c / block, at_r = b * 2 * block + (c - b * block), at_i = at_r + block;
+  const float bias_r = gate_bias[at_r], bias_i = gate_bias[at_i], rt = rate[c], yb = y_bias != nullptr ? y_bias[c] : 0.f;
+  const int row0 = segment_rows[seg], len = segment_lengths[seg];
+  float* sp = state + (int64_t)segment_slots[seg] * W + c;
+  float S = *sp;
+  for (int first = 0; first < len; first += kRgTokens) {
+    float r[kRgTokens], g[kRgTokens], x[kRgTokens], z[kRgTokens];
+#pragma unroll
+    for (int j = 0; j < kRgTokens; ++j) {
+      const bool in = first + j < len;
+      const int64_t row = row0 + first + (in ? j : 0);
+      r[j] = gates[row * ldg + at_r];
+      g[j] = gates[row * ldg + at_i];
+      x[j] = u[row * ldu + c];
+      z[j] = to_float<T>(y[row * ldy + c]);
+    }
+#pragma unroll
+    for (int j = 0; j < kRgTokens; ++j) {
+      const float log_a = rt / (1.0f + expf(-(r[j] + bias_r)));
+      r[j] = expf(log_a);
+      // 1 - a^2 = -(exp(2 log a) - 1): no cancellation where the decay is close to one
+      g[j] = sqrtf(-expm1f(2.0f * log_a)) * x[j] / (1.0f + expf(-(g[j] + bias_i)));
+      const float v = z[j] + yb;
+      z[j] = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+    }
+#pragma unroll
+    for (int j = 0; j < kRgTokens; ++j) {
+      if (first + j < len) {
+        S = fmaf(r[j], S, g[j]);
+        out[(int64_t)(row0 + first + j) * ldo + c] = from_float<T>(S * z[j]);
+      }
+    }
+  }
+  *sp = S;
+}
+
+// One workgroup a (token, part).  o: float32 [n, inner], what the recurrence read; x: float32 [n, inner],
+// the recurrence's input, of which skip[head] times is added; z: the gate's branch in T; weight: float32 [inner].
+template <typename T>
+__global__ __launch_bounds__(256) void gate_group_norm_kernel(
+    T* __restrict__ out, int64_t ldo, const float* __restrict__ o, int64_t ldi, const float* __restrict__ x, int64_t ldx,
+    const float* __restrict__ skip, int head_width, const T* __restrict__ z, int64_t ldz,
+    const float* __restrict__ weight, int part_width, float eps) {
+  __shared__ float scratch[16];
+  const int64_t t = blockIdx.x;
+  const int j0 = blockIdx.y * part_width;
+  float ss = 0.f;
+  for (int j = j0 + threadIdx.x; j < j0 + part_width; j += blockDim.x) {
+    const float g = to_float<T>(z[t * ldz + j]);
+    const float v = fmaf(skip[j / head_width], x[t * ldx + j], o[t * ldi + j]) * (g / (1.0f + expf(-g)));
+    ss = fmaf(v, v, ss);
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)part_width + eps);
+  for (int j = j0 + threadIdx.x; j < j0 + part_width; j += blockDim.x) {
+    const float g = to_float<T>(z[t * ldz + j]);
+    const float v = fmaf(skip[j / head_width], x[t * ldx + j], o[t * ldi + j]) * (g / (1.0f + expf(-g)));
+    out[t * ldo + j] = from_float<T>(v * inv * weight[j]);
+  }
+}
+
 }  // namespace
 
 HFEE_API int hfee_short_conv_silu(float* y, int64_t ldy, const void* x, int64_t ldx, const void* state, int dtype,
                                   const float* taps, const int* token_segment, const int* segment_rows,
-                                  const int* segment_slots, int channels, int taps_count, int n, hipStream_t stream) {
+                                  const int* segment_slots, int channels, int taps_count, int n, const float* in_bias,
+                                  const float* out_bias, int act, hipStream_t stream) {
   HFEE_REQUIRE(n >= 0 && channels > 0 && taps_count >= 1 && taps_count <= 64, "short_conv_silu: bad sizes");
+  HFEE_REQUIRE(act == 0 || act == 1, "short_conv: the activation is none (0) or the SiLU (1)");
   if (n == 0) return 0;
   HFEE_REQUIRE(ldx >= channels && ldy >= channels && (channels + 255) / 256 <= 65535, "short_conv_silu: rows too short or too wide");
   dim3 grid(n, (channels + 255) / 256);
   if (dtype == 0)
     short_conv_silu_kernel<float><<<grid, 256, 0, stream>>>(y, ldy, (const float*)x, ldx, (const float*)state, taps,
-        token_segment, segment_rows, segment_slots, channels, taps_count);
+        token_segment, segment_rows, segment_slots, channels, taps_count, in_bias, out_bias, act);
   else if (dtype == 1)
     short_conv_silu_kernel<bf16_t><<<grid, 256, 0, stream>>>(y, ldy, (const bf16_t*)x, ldx, (const bf16_t*)state, taps,
-        token_segment, segment_rows, segment_slots, channels, taps_count);
+        token_segment, segment_rows, segment_slots, channels, taps_count, in_bias, out_bias, act);
   else
     return fail("short_conv_silu: unknown dtype %d", dtype);
   HFEE_CHECK_LAUNCH("short_conv_silu");
@@ -363,16 +466,16 @@ HFEE_API int hfee_short_conv_silu(float* y, int64_t ldy, const void* x, int64_t 
 
 HFEE_API int hfee_short_conv_keep(void* state, const void* x, int64_t ldx, int dtype, const int* segment_rows,
                                   const int* segment_lengths, const int* segment_slots, int channels, int taps_count,
-                                  int segments, hipStream_t stream) {
+                                  int segments, const float* in_bias, hipStream_t stream) {
   HFEE_REQUIRE(segments >= 0 && segments <= 65535 && channels > 0 && taps_count >= 1, "short_conv_keep: bad sizes");
   if (segments == 0 || taps_count == 1) return 0;
   dim3 grid((channels + 255) / 256, segments);
   if (dtype == 0)
     short_conv_keep_kernel<float><<<grid, 256, 0, stream>>>((float*)state, (const float*)x, ldx, segment_rows,
-        segment_lengths, segment_slots, channels, taps_count);
+        segment_lengths, segment_slots, channels, taps_count, in_bias);
   else if (dtype == 1)
     short_conv_keep_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)state, (const bf16_t*)x, ldx, segment_rows,
-        segment_lengths, segment_slots, channels, taps_count);
+        segment_lengths, segment_slots, channels, taps_count, in_bias);
   else
     return fail("short_conv_keep: unknown dtype %d", dtype);
   HFEE_CHECK_LAUNCH("short_conv_keep");
@@ -392,7 +495,7 @@ HFEE_API int hfee_scan_gate(float* out, int64_t ldo, const void* z, int64_t ldz,
                             const float* per_head, int head_width, int mode, float number, int first_columns, int n,
                             int width, hipStream_t stream) {
   HFEE_REQUIRE(n >= 0 && width > 0 && (width + 255) / 256 <= 65535 && ldo >= width && ldz >= width, "scan_gate: bad sizes");
-  HFEE_REQUIRE(mode >= 0 && mode <= 3, "scan_gate: unknown mode %d", mode);
+  HFEE_REQUIRE(mode >= 0 && mode <= 4, "scan_gate: unknown mode %d", mode);
   HFEE_REQUIRE(mode != 0 || (per_head != nullptr && head_width > 0), "scan_gate: a decay from a step size needs a number a head");
   HFEE_REQUIRE(mode != 1 || number > 0.f, "scan_gate: tau must be positive");
   if (n == 0) return 0;
@@ -413,25 +516,26 @@ HFEE_API int hfee_linear_scan(float* out, int64_t ldo, float* state, const float
                               int64_t ldk, const float* v, int64_t ldv, const float* decay, int64_t ldd,
                               const float* beta, int64_t ldb, const int* segment_rows, const int* segment_lengths,
                               const int* segment_slots, int segments, int heads, int qk_heads, int dim, int vdim,
-                              int rule, hipStream_t stream) {
+                              int rule, int decay_per_head, hipStream_t stream) {
   HFEE_REQUIRE(segments >= 0 && segments <= 65535, "linear_scan: bad segment count");
   if (segments == 0) return 0;
   HFEE_REQUIRE(heads > 0 && qk_heads > 0 && heads % qk_heads == 0 && heads <= 65535,
                "linear_scan: %d heads are not a multiple of %d query/key heads", heads, qk_heads);
   HFEE_REQUIRE(dim >= 1 && dim <= 512 && vdim >= 1, "linear_scan: key sizes of 1 to 512");
-  HFEE_REQUIRE(rule == 0 || (rule == 1 && beta != nullptr), "linear_scan: rule 0, or rule 1 with its writing strengths");
+  HFEE_REQUIRE(rule == 0 || ((rule == 1 || rule == 2) && beta != nullptr && ldb >= heads),
+               "linear_scan: rule 0, or rule 1 or 2 with a number a head and token");
   HFEE_REQUIRE(ldq >= (int64_t)qk_heads * dim && ldk >= (int64_t)qk_heads * dim && ldv >= (int64_t)heads * vdim &&
-               ldd >= (int64_t)heads * dim && ldo >= (int64_t)heads * vdim, "linear_scan: rows too short");
+               ldd >= (decay_per_head ? (int64_t)heads : (int64_t)heads * dim) && ldo >= (int64_t)heads * vdim, "linear_scan: rows too short");
   const int columns = kScanWaves * kScanColumns;
   dim3 grid((vdim + columns - 1) / columns, heads, segments);
   const int per = (dim + kScanParts - 1) / kScanParts;
 #define LAUNCH(DPT, RULE)                                                                                             \
   linear_scan_kernel<DPT, RULE><<<grid, kScanWaves * 64, 2 * ScanShape<DPT>::BUFFER * sizeof(float), stream>>>(out, ldo, state, q, ldq, k, ldk, v, ldv, decay, ldd, beta, ldb, \
-      segment_rows, segment_lengths, segment_slots, heads, qk_heads, dim, vdim)
+      segment_rows, segment_lengths, segment_slots, heads, qk_heads, dim, vdim, decay_per_head)
 #define PICK(RULE)                                                                                                    \
   if (per <= 1) LAUNCH(1, RULE); else if (per <= 2) LAUNCH(2, RULE); else if (per <= 4) LAUNCH(4, RULE);              \
   else if (per <= 8) LAUNCH(8, RULE); else if (per <= 16) LAUNCH(16, RULE); else LAUNCH(32, RULE)
-  if (rule == 0) { PICK(0); } else { PICK(1); }
+  if (rule == 0) { PICK(0); } else if (rule == 1) { PICK(1); } else { PICK(2); }
 #undef PICK
 #undef LAUNCH
   HFEE_CHECK_LAUNCH("linear_scan");
@@ -456,5 +560,47 @@ HFEE_API int hfee_head_norm_gate(void* out, int64_t ldo, const float* o, int64_t
   else
     return fail("head_norm_gate: unknown dtype %d", dtype);
   HFEE_CHECK_LAUNCH("head_norm_gate");
+  return 0;
+}
+
+HFEE_API int hfee_rglru_scan(void* out, int64_t ldo, int dtype, float* state, const float* gates, int64_t ldg,
+                             const float* gate_bias, const float* u, int64_t ldu, const float* rate, const void* y,
+                             int64_t ldy, const float* y_bias, const int* segment_rows, const int* segment_lengths,
+                             const int* segment_slots, int segments, int width, int block, hipStream_t stream) {
+  HFEE_REQUIRE(segments >= 0 && segments <= 65535 && width > 0 && block > 0 && width % block == 0,
+               "rglru_scan: %d channels are not whole blocks of %d", width, block);
+  HFEE_REQUIRE(ldo >= width && ldu >= width && ldy >= width && ldg >= 2 * (int64_t)width, "rglru_scan: rows too short");
+  HFEE_REQUIRE(gate_bias != nullptr && rate != nullptr, "rglru_scan: the gates' biases and the decay's rates");
+  if (segments == 0) return 0;
+  dim3 grid((width + 255) / 256, segments);
+  if (dtype == 0)
+    rglru_scan_kernel<float><<<grid, 256, 0, stream>>>((float*)out, ldo, state, gates, ldg, gate_bias, u, ldu, rate,
+        (const float*)y, ldy, y_bias, segment_rows, segment_lengths, segment_slots, width, block);
+  else if (dtype == 1)
+    rglru_scan_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out, ldo, state, gates, ldg, gate_bias, u, ldu, rate,
+        (const bf16_t*)y, ldy, y_bias, segment_rows, segment_lengths, segment_slots, width, block);
+  else
+    return fail("rglru_scan: unknown dtype %d", dtype);
+  HFEE_CHECK_LAUNCH("rglru_scan");
+  return 0;
+}
+
+HFEE_API int hfee_gate_group_norm(void* out, int64_t ldo, int dtype, const float* o, int64_t ldi, const float* x,
+                                  int64_t ldx, const float* skip, int head_width, const void* z, int64_t ldz,
+                                  const float* weight, int parts, int inner, float eps, int n, hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && inner > 0 && parts > 0 && parts <= 65535 && inner % parts == 0 && head_width > 0 && inner % head_width == 0,
+               "gate_group_norm: %d values are not %d equal parts (or whole heads of %d)", inner, parts, head_width);
+  HFEE_REQUIRE(ldo >= inner && ldi >= inner && ldx >= inner && ldz >= inner && eps >= 0.f, "gate_group_norm: rows too short");
+  if (n == 0) return 0;
+  dim3 grid(n, parts);
+  if (dtype == 0)
+    gate_group_norm_kernel<float><<<grid, 256, 0, stream>>>((float*)out, ldo, o, ldi, x, ldx, skip, head_width,
+        (const float*)z, ldz, weight, inner / parts, eps);
+  else if (dtype == 1)
+    gate_group_norm_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out, ldo, o, ldi, x, ldx, skip, head_width,
+        (const bf16_t*)z, ldz, weight, inner / parts, eps);
+  else
+    return fail("gate_group_norm: unknown dtype %d", dtype);
+  HFEE_CHECK_LAUNCH("gate_group_norm");
   return 0;
 }

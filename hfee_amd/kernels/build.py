@@ -5,7 +5,8 @@ Two kinds of library:
   * `attention_bf16_hd<N>`: the matrix-core attention kernels, compiled for one head
     size each, on demand (a model compiles only the head size it has);
   * `attention_kv_bf16_k<Dk>_v<Dv>`: the matrix-core attention for keys and values of
-    different sizes, compiled per pair of sizes, on demand;
+    different sizes, compiled per pair of sizes, on demand; with `_sigmoid` behind the name
+    the same kernels without a softmax (a key weighs sigmoid(score + a number a head));
   * `attention_mix_bf16_h<H>_g<G>_d<D>`: the matrix-core attention whose heads' scores are mixed,
     compiled per number of heads, of key heads and head size, on demand.
 Libraries are built in-tree (hfee_amd/_lib); if that folder cannot be written, in a
@@ -36,7 +37,7 @@ FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-fvisibility=h
 
 CORE_SOURCES = ["elementwise.hip", "gemm_f32.hip", "attention_ref.hip", "gemm_bf16.hip", "gemm_skinny.hip",
                 "sampling.hip", "random_fill.hip", "yardstick.hip", "attention_kv.hip", "rowwise.hip", "attention_mix.hip",
-                "recurrent.hip", "moe.hip"]
+                "recurrent.hip", "moe.hip", "gated_rows.hip"]
 ATTENTION_SOURCE = "attention_bf16.hip"
 HEAD_DIMS = tuple(range(16, 257, 16))
 ATTENTION_KV_SOURCE = "attention_kv_bf16.hip"      # compiled per (key size, value size)
@@ -57,6 +58,8 @@ def attention_mix_fits(heads: int, dim: int) -> bool:
 # the pairs that `build_all` compiles: those of the tests and of bench.py's comparison (a model with
 # other sizes compiles its own at first use)
 ATTENTION_KV_SIZES = ((32, 16), (64, 32), (96, 64), (48, 32), (16, 48), (112, 96), (64, 64), (160, 128), (128, 128), (576, 512))
+# the same for the kernels without a softmax
+ATTENTION_KV_SIGMOID_SIZES = ((32, 16), (16, 48), (32, 64), (128, 128))
 
 
 class BuildError(RuntimeError):
@@ -122,14 +125,17 @@ def library_spec(name: str):
                              f"in steps of 16, not {hd}")
         return [ATTENTION_SOURCE], [f"-DHFEE_HEAD_DIM={hd}"]
     if name.startswith("attention_kv_bf16_k"):
+        sizes, weights = name[len("attention_kv_bf16_k"):], 0
+        if sizes.endswith("_sigmoid"):
+            sizes, weights = sizes[:-len("_sigmoid")], 1
         try:
-            dk, dv = (int(n) for n in name[len("attention_kv_bf16_k"):].split("_v"))
+            dk, dv = (int(n) for n in sizes.split("_v"))
         except ValueError:
             raise BuildError(f"unknown kernel library {name!r}") from None
         if dk % 16 or dv % 16 or not 16 <= dk <= ATTENTION_KV_MOST[0] or not 16 <= dv <= ATTENTION_KV_MOST[1]:
             raise BuildError(f"the attention kernels for keys and values of different sizes take multiples of 16 up to "
                              f"{ATTENTION_KV_MOST}, not ({dk}, {dv})")
-        return [ATTENTION_KV_SOURCE], [f"-DHFEE_DK={dk}", f"-DHFEE_DV={dv}"]
+        return [ATTENTION_KV_SOURCE], [f"-DHFEE_DK={dk}", f"-DHFEE_DV={dv}"] + (["-DHFEE_KV_WEIGHTS=1"] if weights else [])
     if name.startswith("attention_mix_bf16_h"):
         try:
             heads, rest = name[len("attention_mix_bf16_h"):].split("_g")
@@ -213,13 +219,15 @@ def build_library(name: str, force: bool = False) -> str:
     return so
 
 
-def build_all(head_dims=HEAD_DIMS, force: bool = True, kv_sizes=ATTENTION_KV_SIZES, mix_sizes=ATTENTION_MIX_SIZES) -> list:
+def build_all(head_dims=HEAD_DIMS, force: bool = True, kv_sizes=ATTENTION_KV_SIZES, mix_sizes=ATTENTION_MIX_SIZES,
+              kv_sigmoid_sizes=ATTENTION_KV_SIGMOID_SIZES) -> list:
     """Compiles the core library, the attention library of every head size, and the attention
     libraries for keys and values of different sizes of the listed pairs."""
     out = [build_library("core", force=force)]
     # the attention libraries are independent: build them side by side
     names = [f"attention_bf16_hd{hd}" for hd in head_dims] + [f"attention_kv_bf16_k{dk}_v{dv}" for dk, dv in kv_sizes]
     names += [f"attention_mix_bf16_h{h}_g{g}_d{d}" for h, g, d in mix_sizes]
+    names += [f"attention_kv_bf16_k{dk}_v{dv}_sigmoid" for dk, dv in kv_sigmoid_sizes]
     errors = []
 
     def work(n):

@@ -48,21 +48,28 @@ _CORE_SIGNATURES = {
     "hfee_read_stream": [P, L, P, I, I, P],
     "hfee_mfma_loop": [P, I, I, P],
     "hfee_kv_write": [P, L, I, I, I, P, L, I, P, L, P, I, P, I, P, P, P, I, P, P, I, I, I, P, I, I, I, I, I, P],
-    "hfee_attention_kv_plain": [P, L, P, L, P, I, P, P, P, I, I, I, I, I, I, F, P, I, P],
+    "hfee_attention_kv_plain": [P, L, P, L, P, I, P, P, P, I, I, I, I, I, I, F, P, I, I, P],
+    "hfee_qk_norm_write": [P, L, I, P, L, P, L, I, P, P, F, F, I, P, P, P, I, P, I, I, I, I, I, P],
     "hfee_head_linear": [P, L, L, P, L, L, P, I, I, I, I, I, I, P],
     "hfee_norm_add": [P, P, I, P, I, P, I, F, F, P, I, P, F, I, I, P],
     "hfee_bias_act": [P, L, P, L, P, I, I, I, I, F, F, P],
     "hfee_layernorm": [P, I, P, P, I, P, F, I, I, P],
     "hfee_attention_mix_prepare": [P, L, P, L, I, I, I, I, P, P, P, I, P, P, I, I, I, I, F, P, I, I, P],
     "hfee_attention_mix": [P, L, P, L, P, I, P, P, P, I, I, I, I, I, F, P, I, I, P, I, P],
-    "hfee_short_conv_silu": [P, L, P, L, P, I, P, P, P, P, I, I, I, P],
-    "hfee_short_conv_keep": [P, P, L, I, P, P, P, I, I, I, P],
+    "hfee_short_conv_silu": [P, L, P, L, P, I, P, P, P, P, I, I, I, P, P, I, P],
+    "hfee_short_conv_keep": [P, P, L, I, P, P, P, I, I, I, P, P],
     "hfee_unit_heads": [P, L, I, I, F, F, I, P],
     "hfee_scan_gate": [P, L, P, L, I, P, P, I, I, F, I, I, I, P],
-    "hfee_linear_scan": [P, L, P, P, L, P, L, P, L, P, L, P, L, P, P, P, I, I, I, I, I, I, P],
+    "hfee_linear_scan": [P, L, P, P, L, P, L, P, L, P, L, P, L, P, P, P, I, I, I, I, I, I, I, P],
+    "hfee_rglru_scan": [P, L, I, P, P, L, P, P, L, P, P, L, P, P, P, P, I, I, I, P],
+    "hfee_gate_group_norm": [P, L, I, P, L, P, L, P, I, P, L, P, I, I, F, I, P],
+    "hfee_router_topk": [P, L, I, I, I, P, P, P],
+    "hfee_add_table_rows": [P, I, I, P, I, P, P],
+    "hfee_scaled_add": [P, P, F, P, F, L, P],
+    "hfee_gated_norm_add": [P, P, P, F, F, P, I, L, P, P, F, P, I, P, F, I, I, P],
     "hfee_head_norm_gate": [P, L, P, L, P, L, I, P, I, I, F, I, I, P],
-    "hfee_moe_grouped": [P, L, P, L, P, P, P, P, P, P, P, F, I, I, I, I, I, P, P, P, P, P],
-    "hfee_moe_up": [P, P, L, P, P, I, P, P, P, I, I, I, I, I, P],
+    "hfee_moe_grouped": [P, L, P, L, P, P, P, P, P, P, P, F, I, I, I, I, I, P, P, P, P, P, P],
+    "hfee_moe_up": [P, P, L, P, P, I, P, P, P, I, I, I, I, I, P, P],
     "hfee_moe_down": [P, L, P, P, I, P, P, P, P, F, I, I, I, I, I, I, P],
     "hfee_rmsnorm_cols": [P, L, P, L, I, P, I, F, F, I, I, P],
 }
@@ -70,6 +77,7 @@ _CORE_SIGNATURES = {
 _ATTENTION_KV_SIGNATURES = {
     "hfee_attention_kv_bf16_dk": [],
     "hfee_attention_kv_bf16_dv": [],
+    "hfee_attention_kv_bf16_weights": [],
     "hfee_attention_kv_bf16_rows": [I],
     "hfee_attention_kv_bf16": [P, L, P, L, P, P, I, I, P, I, I, I, I, F, P, P, L, I, P],
 }
@@ -148,12 +156,15 @@ def attention_bf16(head_dim: int) -> Library:
     return load(f"attention_bf16_hd{head_dim}")
 
 
-def attention_kv_bf16(dk: int, dv: int) -> Library:
-    """The matrix-core attention for keys of dk and values of dv dims (multiples of 16)."""
+def attention_kv_bf16(dk: int, dv: int, weights: str = "softmax") -> Library:
+    """The matrix-core attention for keys of dk and values of dv dims (multiples of 16); weights
+    "softmax", or "sigmoid" for the kernels in which a key weighs sigmoid(score + a number a head)."""
+    if weights not in ("softmax", "sigmoid"):
+        raise KernelError(f'the weights of a key are a "softmax"\'s or a "sigmoid", not {weights!r}')
     if dk % 16 or dv % 16 or dk < 16 or dv < 16:
         raise KernelError(f"the bfloat16 attention kernels for keys and values of different sizes take multiples "
                           f"of 16, not ({dk}, {dv})")
-    return load(f"attention_kv_bf16_k{dk}_v{dv}")
+    return load(f"attention_kv_bf16_k{dk}_v{dv}" + ("_sigmoid" if weights == "sigmoid" else ""))
 
 
 def attention_mix_bf16(heads: int, kv_heads: int, dim: int) -> Library:

@@ -846,10 +846,15 @@ def kv_write(q, k, v, positions, token_segment, block_tables, cos, sin, cache_la
                     int(max_position), _ptr(cache_layer if has_k else None), kv_heads, dk, dv, page_size, n, _stream())
 
 
+KEY_WEIGHTS = {"softmax": 0, "sigmoid": 1}
+
+
 def attention_kv_plain(out, q, cache_layer, positions, token_segment, block_tables, num_heads: int, kv_heads: int,
-                       dk: int, dv: int, page_size: int, scale: float, sinks=None):
+                       dk: int, dv: int, page_size: int, scale: float, sinks=None, weights: str = "softmax"):
     """One wave per (token, head), any sizes, both dtypes: token t of head h reads the keys
-    0..pos of its sequence; `sinks` (float32 [num_heads] or None) joins the softmax's denominator."""
+    0..pos of its sequence; `sinks` (float32 [num_heads] or None) joins the softmax's denominator.
+    weights "sigmoid": no softmax, a key weighs sigmoid(score + sinks[head]) and nothing is normalized."""
+    _check(weights in KEY_WEIGHTS, f"attention_kv: the weights are {sorted(KEY_WEIGHTS)}, not {weights!r}")
     _gpu(out, q, cache_layer, positions, token_segment, block_tables, sinks)
     n, w, ldq = _rows2d(q, "attention_kv q")
     no, wo, ldo = _rows2d(out, "attention_kv out")
@@ -865,7 +870,37 @@ def attention_kv_plain(out, q, cache_layer, positions, token_segment, block_tabl
                "attention_kv: sinks must be float32 [num_heads]")
     lib.core().call("hfee_attention_kv_plain", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), _dt(q),
                     _ptr(positions), _ptr(token_segment), _ptr(block_tables), block_tables.stride(0),
-                    num_heads, kv_heads, dk, dv, page_size, float(scale), _ptr(sinks), n, _stream())
+                    num_heads, kv_heads, dk, dv, page_size, float(scale), _ptr(sinks), KEY_WEIGHTS[weights], n, _stream())
+
+
+def qk_norm_write(q, k, v, positions, token_segment, block_tables, cache_layer, q_weight, k_weight, eps: float,
+                  num_heads: int, kv_heads: int, dk: int, dv: int, page_size: int, temperature=None):
+    """q (in place) and k (into the cache) are divided by their root mean square over each head and
+    multiplied by q_weight / k_weight (float32 [dk], shared by the heads); v goes into the cache as it is.
+    temperature (coef, every): q is also multiplied by 1 + coef * ln(floor((p + 1) / every) + 1) at
+    position p.  k and v None: the queries only."""
+    _gpu(q, k, v, positions, token_segment, block_tables, cache_layer, q_weight, k_weight)
+    n, wq, ldq = _rows2d(q, "qk_norm_write q")
+    _check(wq == num_heads * dk, "qk_norm_write: q width")
+    _check(q_weight.dtype == torch.float32 and q_weight.is_contiguous() and q_weight.numel() == dk, "qk_norm_write: q_weight float32 [dk]")
+    _i32(positions, "qk_norm_write positions", n)
+    ldk = ldv = 0
+    if k is not None:
+        nk, wk, ldk = _rows2d(k, "qk_norm_write k")
+        nv, wv, ldv = _rows2d(v, "qk_norm_write v")
+        _check(nk == nv == n and wk == kv_heads * dk and wv == kv_heads * dv and k.dtype == v.dtype == q.dtype == cache_layer.dtype,
+               "qk_norm_write: k/v shapes and dtypes")
+        _check(k_weight is not None and k_weight.dtype == torch.float32 and k_weight.is_contiguous() and k_weight.numel() == dk,
+               "qk_norm_write: k_weight float32 [dk]")
+        _kv_cache(cache_layer, kv_heads, dk, dv, page_size, "qk_norm_write")
+        _i32(token_segment, "qk_norm_write token_segment", n)
+        _check(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.stride(1) == 1, "qk_norm_write: block tables")
+    coef, every = (float(temperature[0]), int(temperature[1])) if temperature else (0.0, 0)
+    _check(every >= 0, "qk_norm_write: the temperature's step must be positive")
+    lib.core().call("hfee_qk_norm_write", _ptr(q), ldq, num_heads, _ptr(k), ldk, _ptr(v), ldv, _dt(q), _ptr(q_weight),
+                    _ptr(k_weight), float(eps), coef, every, _ptr(positions), _ptr(token_segment), _ptr(block_tables),
+                    block_tables.stride(0) if k is not None else 0, _ptr(cache_layer if k is not None else None),
+                    kv_heads, dk, dv, page_size, n, _stream())
 
 
 def attention_kv_sizes_fit(dk: int, dv: int) -> bool:
@@ -874,10 +909,10 @@ def attention_kv_sizes_fit(dk: int, dv: int) -> bool:
     return dk % 16 == 0 and dv % 16 == 0 and 16 <= dk <= build.ATTENTION_KV_MOST[0] and 16 <= dv <= build.ATTENTION_KV_MOST[1]
 
 
-def attention_kv_rows(dk: int, dv: int, heads_per_kv_head: int = 1) -> int:
+def attention_kv_rows(dk: int, dv: int, heads_per_kv_head: int = 1, weights: str = "softmax") -> int:
     """The most rows that an item of `attention_kv_bf16`'s mode 0 may hold for these sizes and this
     many query heads a key/value head."""
-    return int(lib.attention_kv_bf16(dk, dv).raw("hfee_attention_kv_bf16_rows")(int(heads_per_kv_head)))
+    return int(lib.attention_kv_bf16(dk, dv, weights).raw("hfee_attention_kv_bf16_rows")(int(heads_per_kv_head)))
 
 
 def attention_kv_partial_words(num_items: int, num_heads: int, dv: int, splits: int) -> int:
@@ -885,8 +920,9 @@ def attention_kv_partial_words(num_items: int, num_heads: int, dv: int, splits: 
 
 
 def attention_kv_bf16(out, q, cache_layer, items, mode: int, block_tables, num_heads: int, kv_heads: int, dk: int,
-                      dv: int, page_size: int, scale: float, sinks=None, partial=None, splits: int = 1):
-    """Matrix-core attention, bfloat16.  items: int32 [count, 4] on the device (first row, rows,
+                      dv: int, page_size: int, scale: float, sinks=None, partial=None, splits: int = 1,
+                      weights: str = "softmax"):
+    """Matrix-core attention, bfloat16 (weights: as in `attention_kv_plain`).  items: int32 [count, 4] on the device (first row, rows,
     first position, block-table row).  mode 0: an item is up to `attention_kv_rows` consecutive tokens of a portion;
     mode 1: an item is a single token (rows = 1), whose keys may be split over `splits` waves that
     leave partial results in `partial` (float32, `attention_kv_partial_words`) for a joining kernel."""
@@ -905,7 +941,7 @@ def attention_kv_bf16(out, q, cache_layer, items, mode: int, block_tables, num_h
                "attention_kv: sinks must be float32 [num_heads]")
     if partial is not None:
         _check(partial.dtype == torch.float32 and partial.is_contiguous(), "attention_kv: float32 partial buffer expected")
-    lib.attention_kv_bf16(dk, dv).call(
+    lib.attention_kv_bf16(dk, dv, weights).call(
         "hfee_attention_kv_bf16", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), _ptr(items), items.shape[0], int(mode),
         _ptr(block_tables), block_tables.stride(0), num_heads, kv_heads, page_size, float(scale), _ptr(sinks),
         _ptr(partial), 0 if partial is None else partial.numel(), int(splits), _stream())
@@ -952,6 +988,52 @@ def norm_add(x, y, weight, eps: float, bias=None, next_out=None, next_weight=Non
     lib.core().call("hfee_norm_add", _ptr(x), _ptr(y), _dt(y), _ptr(bias), 0 if bias is None else _dt(bias),
                     _ptr(weight), _dt(weight), 0.0, float(eps), _ptr(next_out), 0 if next_out is None else _dt(next_out),
                     _ptr(next_weight), float(next_eps), n, d, _stream())
+
+
+def add_table_rows(x, table, index):
+    """x[r] (float32 [n, d]) += table[index[r]] (a learned vector a position, a segment, ...)."""
+    _gpu(x, table, index)
+    n, d, _ = _rows2d(x, "add_table_rows x")
+    _check(x.dtype == torch.float32 and x.is_contiguous() and table.dim() == 2 and table.is_contiguous() and table.shape[1] == d,
+           "add_table_rows: contiguous float32 x and a table of its width")
+    _i32(index, "add_table_rows index", n)
+    lib.core().call("hfee_add_table_rows", _ptr(x), n, d, _ptr(table), _dt(table), _ptr(index), _stream())
+
+
+def scaled_add(x, y, a: float = 1.0, y2=None, b: float = 1.0):
+    """x += a * y + b * y2 (y2 optional); float32, contiguous, one shape."""
+    _gpu(x, y, y2)
+    _check(x.dtype == y.dtype == torch.float32 and x.is_contiguous() and y.is_contiguous() and x.shape == y.shape,
+           "scaled_add: contiguous float32 x and y of one shape")
+    if y2 is not None:
+        _check(y2.dtype == torch.float32 and y2.is_contiguous() and y2.shape == x.shape, "scaled_add: y2 like y")
+    lib.core().call("hfee_scaled_add", _ptr(x), _ptr(y), float(a), _ptr(y2), float(b), x.numel(), _stream())
+
+
+def gated_norm_add(x, y, weight, eps: float, y2=None, scales=(1.0, 1.0), gate=None, gate_bias=None, next_out=None,
+                   next_weight=None, next_eps: float = 0.0):
+    """With v = (scales[0] * y + scales[1] * y2) * sigmoid(gate + gate_bias) (y2 and the gate optional):
+    x (float32, the residual stream) += v / sqrt(mean(v^2) + eps) * weight; with next_out also
+    next_out = norm(x_new) * next_weight (eps next_eps).  y, y2 float32 [n, d] contiguous; gate [n, d] in
+    either dtype (rows of a wider buffer allowed); the weights and the gate's bias float32."""
+    _gpu(x, y, weight, y2, gate, gate_bias, next_out, next_weight)
+    n, d, _ = _rows2d(x, "gated_norm_add x")
+    _check(x.dtype == y.dtype == torch.float32 and x.is_contiguous() and y.is_contiguous() and tuple(y.shape) == (n, d),
+           "gated_norm_add: contiguous float32 x and y of one shape")
+    if y2 is not None:
+        _check(y2.dtype == torch.float32 and y2.is_contiguous() and tuple(y2.shape) == (n, d), "gated_norm_add: y2 like y")
+    ldg = 0
+    if gate is not None:
+        ng, wg, ldg = _rows2d(gate, "gated_norm_add gate")
+        _check(ng == n and wg == d, "gated_norm_add: gate shape")
+    for t, what in ((weight, "weight"), (gate_bias, "gate_bias"), (next_weight, "next_weight")):
+        if t is not None:
+            _check(t.dtype == torch.float32 and t.is_contiguous() and t.numel() == d, f"gated_norm_add: {what} float32 [d]")
+    if next_out is not None:
+        _check(next_weight is not None and next_out.is_contiguous() and tuple(next_out.shape) == (n, d), "gated_norm_add: next_out")
+    lib.core().call("hfee_gated_norm_add", _ptr(x), _ptr(y), _ptr(y2), float(scales[0]), float(scales[1]), _ptr(gate),
+                    0 if gate is None else _dt(gate), ldg, _ptr(gate_bias), _ptr(weight), float(eps), _ptr(next_out),
+                    0 if next_out is None else _dt(next_out), _ptr(next_weight), float(next_eps), n, d, _stream())
 
 
 def bias_act(out, x, bias, activation: str = "none", numbers=(0.0, 0.0)):
@@ -1136,11 +1218,18 @@ def _f32rows(t, what):
     return n, w, ld
 
 
-def short_conv_silu(y, x, state, taps, token_segment, segment_rows, segment_slots):
+def short_conv_silu(y, x, state, taps, token_segment, segment_rows, segment_slots, in_bias=None, out_bias=None,
+                    activation: str = "silu"):
     """y (float32 [n, C]) = silu of the causal convolution of x ([n, C], the step's rows) with taps
     (float32 [C, K], the last column the current token's) per channel; the K - 1 inputs before a
-    portion's first token come from state[slot] ([slots, K - 1, C] in x's dtype, the newest last)."""
-    _gpu(y, x, state, taps, token_segment, segment_rows, segment_slots)
+    portion's first token come from state[slot] ([slots, K - 1, C] in x's dtype, the newest last).
+    in_bias (float32 [C]) is added to every input that exists (before a sequence's start stand zeros),
+    out_bias (float32 [C]) to the sum; activation "silu" or "none"."""
+    _gpu(y, x, state, taps, token_segment, segment_rows, segment_slots, in_bias, out_bias)
+    _check(activation in ("silu", "none"), "short_conv: the activation is 'silu' or 'none'")
+    for b in (in_bias, out_bias):
+        if b is not None:
+            _check(b.dtype == torch.float32 and b.is_contiguous() and b.numel() == x.shape[1], "short_conv: a bias is float32 [C]")
     n, C, ldx = _rows2d(x, "short_conv_silu x")
     ny, wy, ldy = _f32rows(y, "short_conv_silu y")
     K = taps.shape[1]
@@ -1152,13 +1241,16 @@ def short_conv_silu(y, x, state, taps, token_segment, segment_rows, segment_slot
     _i32(segment_rows, "short_conv_silu segment_rows")
     _i32(segment_slots, "short_conv_silu segment_slots")
     lib.core().call("hfee_short_conv_silu", _ptr(y), ldy, _ptr(x), ldx, _ptr(state), _dt(x), _ptr(taps),
-                    _ptr(token_segment), _ptr(segment_rows), _ptr(segment_slots), C, K, n, _stream())
+                    _ptr(token_segment), _ptr(segment_rows), _ptr(segment_slots), C, K, n, _ptr(in_bias), _ptr(out_bias),
+                    1 if activation == "silu" else 0, _stream())
 
 
-def short_conv_keep(state, x, segment_rows, segment_lengths, segment_slots):
-    """state[slot] <- the last K - 1 inputs of each segment's sequence (the step's rows x, and what the
-    state held before where a portion is shorter than K - 1)."""
-    _gpu(state, x, segment_rows, segment_lengths, segment_slots)
+def short_conv_keep(state, x, segment_rows, segment_lengths, segment_slots, in_bias=None):
+    """state[slot] <- the last K - 1 inputs of each segment's sequence (the step's rows x with in_bias,
+    and what the state held before where a portion is shorter than K - 1)."""
+    _gpu(state, x, segment_rows, segment_lengths, segment_slots, in_bias)
+    if in_bias is not None:
+        _check(in_bias.dtype == torch.float32 and in_bias.is_contiguous() and in_bias.numel() == x.shape[1], "short_conv_keep: in_bias float32 [C]")
     n, C, ldx = _rows2d(x, "short_conv_keep x")
     _check(state.dtype == x.dtype and state.is_contiguous() and state.dim() == 3 and state.shape[2] == C,
            "short_conv_keep: the state must be [slots, K - 1, C] in x's dtype")
@@ -1167,7 +1259,7 @@ def short_conv_keep(state, x, segment_rows, segment_lengths, segment_slots):
     _i32(segment_lengths, "short_conv_keep segment_lengths", segments)
     _i32(segment_slots, "short_conv_keep segment_slots", segments)
     lib.core().call("hfee_short_conv_keep", _ptr(state), _ptr(x), ldx, _dt(x), _ptr(segment_rows), _ptr(segment_lengths),
-                    _ptr(segment_slots), C, state.shape[1] + 1, segments, _stream())
+                    _ptr(segment_slots), C, state.shape[1] + 1, segments, _ptr(in_bias), _stream())
 
 
 def unit_heads(x, heads: int, dim: int, eps: float, factor: float = 1.0):
@@ -1178,14 +1270,14 @@ def unit_heads(x, heads: int, dim: int, eps: float, factor: float = 1.0):
     lib.core().call("hfee_unit_heads", _ptr(x), ldx, heads, dim, float(eps), float(factor), n, _stream())
 
 
-SCAN_GATES = {"step_decay": 0, "root_sigmoid": 1, "sigmoid": 2, "cast": 3}
+SCAN_GATES = {"step_decay": 0, "root_sigmoid": 1, "sigmoid": 2, "cast": 3, "softplus": 4}
 
 
 def scan_gate(out, z, kind: str, bias=None, per_head=None, head_width: int = 0, number: float = 1.0, first_columns: int = 0):
     """out (float32) from a projection z (engine dtype), column by column:
     "step_decay": exp(-exp(per_head[column // head_width]) * softplus(z + bias));
     "root_sigmoid": sigmoid(z + bias) ** (1 / number);  "sigmoid": sigmoid(z + bias);
-    "cast": z * number in the first `first_columns` columns, z in the others."""
+    "cast": z * number in the first `first_columns` columns, z in the others;  "softplus": softplus(z + bias)."""
     _gpu(out, z, bias, per_head)
     n, w, ldz = _rows2d(z, "scan_gate z")
     no, wo, ldo = _f32rows(out, "scan_gate out")
@@ -1222,24 +1314,27 @@ def scan_state_matrix(state: torch.Tensor, dim: int, vdim: int) -> torch.Tensor:
 
 
 def linear_scan(out, state, q, k, v, decay, beta, segment_rows, segment_lengths, segment_slots, heads: int,
-                qk_heads: int, dim: int, vdim: int, rule: str):
+                qk_heads: int, dim: int, vdim: int, rule: str, decay_per_head: bool = False):
     """Walks each segment's rows in order from state[slot] (float32 [slots, heads, `scan_state_shape`],
     updated in place: a head's matrix in blocks of four columns).  rule "decay_add": S <- diag(decay) S + k v^T; "delta": S <- diag(decay) S,
-    S <- S + k (beta (v - S^T k))^T; out = S^T q.  q, k: float32 [n, qk_heads * dim] (head h reads
-    q/k head h // (heads / qk_heads)); v, out: [n, heads * vdim]; decay: [n, heads * dim]; beta [n, heads]."""
+    S <- S + k (beta (v - S^T k))^T; "scaled_add": S <- diag(decay) S + k (beta v)^T; out = S^T q.
+    q, k: float32 [n, qk_heads * dim] (head h reads q/k head h // (heads / qk_heads)); v, out:
+    [n, heads * vdim]; decay: [n, heads * dim], or with decay_per_head [n, heads], one number for all
+    of a head's rows; beta [n, heads]."""
     _gpu(out, state, q, k, v, decay, beta, segment_rows, segment_lengths, segment_slots)
     n, wq, ldq = _f32rows(q, "linear_scan q")
     nk, wk, ldk = _f32rows(k, "linear_scan k")
     nv, wv, ldv = _f32rows(v, "linear_scan v")
     nd, wd, ldd = _f32rows(decay, "linear_scan decay")
     no, wo, ldo = _f32rows(out, "linear_scan out")
-    _check(rule in ("decay_add", "delta"), "linear_scan: rule is 'decay_add' or 'delta'")
-    _check(nk == nv == nd == no == n and wq == wk == qk_heads * dim and wv == wo == heads * vdim and wd == heads * dim,
-           "linear_scan: shapes")
+    rules = {"decay_add": 0, "delta": 1, "scaled_add": 2}
+    _check(rule in rules, f"linear_scan: rule is one of {sorted(rules)}")
+    _check(nk == nv == nd == no == n and wq == wk == qk_heads * dim and wv == wo == heads * vdim
+           and wd == (heads if decay_per_head else heads * dim), "linear_scan: shapes")
     _check(state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (heads, *scan_state_shape(dim, vdim)),
            "linear_scan: the state must be float32 [slots, heads, *scan_state_shape(dim, vdim)]")
     ldb = 0
-    if rule == "delta":
+    if rule != "decay_add":
         nb, wb, ldb = _f32rows(beta, "linear_scan beta")
         _check(nb == n and wb == heads, "linear_scan: beta [n, heads]")
     segments = segment_rows.numel()
@@ -1247,8 +1342,50 @@ def linear_scan(out, state, q, k, v, decay, beta, segment_rows, segment_lengths,
     _i32(segment_lengths, "linear_scan segment_lengths", segments)
     _i32(segment_slots, "linear_scan segment_slots", segments)
     lib.core().call("hfee_linear_scan", _ptr(out), ldo, _ptr(state), _ptr(q), ldq, _ptr(k), ldk, _ptr(v), ldv, _ptr(decay),
-                    ldd, _ptr(beta if rule == "delta" else None), ldb, _ptr(segment_rows), _ptr(segment_lengths),
-                    _ptr(segment_slots), segments, heads, qk_heads, dim, vdim, 1 if rule == "delta" else 0, _stream())
+                    ldd, _ptr(beta if rule != "decay_add" else None), ldb, _ptr(segment_rows), _ptr(segment_lengths),
+                    _ptr(segment_slots), segments, heads, qk_heads, dim, vdim, rules[rule], 1 if decay_per_head else 0, _stream())
+
+
+def rglru_scan(out, state, gates, gate_bias, u, rate, y, y_bias, segment_rows, segment_lengths, segment_slots, block: int):
+    """The real-gated linear recurrent unit, a number a channel: with r, i the gates of a token (gates:
+    float32 [n, blocks, 2 * block] before bias and sigmoid, a block's r, then its i; gate_bias float32 of
+    that width), a = exp(rate * sigmoid(r)) (rate float32 [W], not positive),
+    S <- a S + sqrt(1 - a^2) sigmoid(i) u, out = S * gelu_tanh(y + y_bias) in y's dtype.  state: float32
+    [slots, W], walked from and left in each segment's slot; u float32 [n, W]; y [n, W]."""
+    _gpu(out, state, gates, gate_bias, u, rate, y, y_bias, segment_rows, segment_lengths, segment_slots)
+    n, W, ldu = _f32rows(u, "rglru_scan u")
+    ng, wg, ldg = _f32rows(gates, "rglru_scan gates")
+    ny, wy, ldy = _rows2d(y, "rglru_scan y")
+    no, wo, ldo = _rows2d(out, "rglru_scan out")
+    _check(ng == ny == no == n and wg == 2 * W and wy == wo == W and out.dtype == y.dtype and W % block == 0, "rglru_scan: shapes")
+    _check(state.dtype == torch.float32 and state.is_contiguous() and state.dim() == 2 and state.shape[1] == W, "rglru_scan: state float32 [slots, W]")
+    for t, w, what in ((gate_bias, 2 * W, "gate_bias"), (rate, W, "rate"), (y_bias, W, "y_bias")):
+        if t is not None:
+            _check(t.dtype == torch.float32 and t.is_contiguous() and t.numel() == w, f"rglru_scan: {what} float32 [{w}]")
+    segments = segment_rows.numel()
+    _i32(segment_rows, "rglru_scan segment_rows")
+    _i32(segment_lengths, "rglru_scan segment_lengths", segments)
+    _i32(segment_slots, "rglru_scan segment_slots", segments)
+    lib.core().call("hfee_rglru_scan", _ptr(out), ldo, _dt(out), _ptr(state), _ptr(gates), ldg, _ptr(gate_bias), _ptr(u), ldu,
+                    _ptr(rate), _ptr(y), ldy, _ptr(y_bias), _ptr(segment_rows), _ptr(segment_lengths), _ptr(segment_slots),
+                    segments, W, int(block), _stream())
+
+
+def gate_group_norm(out, o, x, skip, z, weight, heads: int, parts: int, eps: float):
+    """out = norm((o + skip[head] * x) * silu(z)) * weight, the norm (root mean square, eps) over each of
+    `parts` equal parts of a row; o, x float32 [n, inner], skip float32 [heads], z and out in the engine's
+    dtype, weight float32 [inner]."""
+    _gpu(out, o, x, skip, z, weight)
+    n, inner, ldi = _f32rows(o, "gate_group_norm o")
+    nx, wx, ldx = _f32rows(x, "gate_group_norm x")
+    nz, wz, ldz = _rows2d(z, "gate_group_norm z")
+    no, wo, ldo = _rows2d(out, "gate_group_norm out")
+    _check(nx == nz == no == n and wx == wz == wo == inner and z.dtype == out.dtype and inner % heads == 0 and inner % parts == 0,
+           "gate_group_norm: shapes")
+    _check(skip.dtype == weight.dtype == torch.float32 and skip.is_contiguous() and weight.is_contiguous()
+           and skip.numel() == heads and weight.numel() == inner, "gate_group_norm: skip float32 [heads], weight float32 [inner]")
+    lib.core().call("hfee_gate_group_norm", _ptr(out), ldo, _dt(out), _ptr(o), ldi, _ptr(x), ldx, _ptr(skip), inner // heads,
+                    _ptr(z), ldz, _ptr(weight), int(parts), inner, float(eps), n, _stream())
 
 
 def head_norm_gate(out, o, gate, weight, heads: int, vdim: int, eps: float, activation: str):
@@ -1276,18 +1413,39 @@ def _experts_of(chosen, table, token_ids, n, top, what):
     _i32(token_ids, f"{what} token_ids", n)
 
 
-def moe_up(act, h, w_gate, w_up, top: int, chosen=None, table=None, token_ids=None):
+def _in_weights(in_weights, w_gate, n, top, what):
+    if in_weights is not None:
+        _check(w_gate is None, f"{what}: only experts without a gate take a weight on their input")
+        _check(in_weights.dtype == torch.float32 and in_weights.is_contiguous() and tuple(in_weights.shape) == (n, top),
+               f"{what}: in_weights float32 [n, top]")
+
+
+def moe_up(act, h, w_gate, w_up, top: int, chosen=None, table=None, token_ids=None, in_weights=None):
     """act[t * top + j] = silu(w_gate[e] @ h[t]) * (w_up[e] @ h[t]), e the j-th expert of token t
-    (chosen[t, j], or table[token_ids[t], j]); w_gate, w_up: [experts, ff, width]."""
-    _gpu(act, h, w_gate, w_up, chosen, table, token_ids)
+    (chosen[t, j], or table[token_ids[t], j]); w_gate, w_up: [experts, ff, width].  w_gate None: experts
+    without a gate, act = relu(in_weights[t, j] * (w_up[e] @ h[t]))^2 (in_weights float32 or None for one)."""
+    _gpu(act, h, w_gate, w_up, chosen, table, token_ids, in_weights)
     n, width, ldh = _rows2d(h, "moe_up h")
-    E, F, W = w_gate.shape
-    _check(W == width and w_up.shape == w_gate.shape and w_gate.is_contiguous() and w_up.is_contiguous(), "moe_up: weights [experts, ff, width]")
-    _check(act.is_contiguous() and tuple(act.shape) == (n * top, F) and act.dtype == h.dtype == w_gate.dtype == w_up.dtype,
+    E, F, W = w_up.shape
+    _check(W == width and w_up.is_contiguous() and (w_gate is None or (w_gate.shape == w_up.shape and w_gate.is_contiguous()
+                                                                      and w_gate.dtype == w_up.dtype)),
+           "moe_up: weights [experts, ff, width]")
+    _check(act.is_contiguous() and tuple(act.shape) == (n * top, F) and act.dtype == h.dtype == w_up.dtype,
            "moe_up: act [n * top, ff], one dtype")
     _experts_of(chosen, table, token_ids, n, top, "moe_up")
+    _in_weights(in_weights, w_gate, n, top, "moe_up")
     lib.core().call("hfee_moe_up", _ptr(act), _ptr(h), ldh, _ptr(w_gate), _ptr(w_up), _dt(h), _ptr(chosen), _ptr(table),
-                    _ptr(token_ids), top, E, F, width, n, _stream())
+                    _ptr(token_ids), top, E, F, width, n, _ptr(in_weights), _stream())
+
+
+def router_topk(chosen, weights, logits, top: int):
+    """chosen (int32 [n, top]) = the experts with the `top` largest scores sigmoid(logits) of each row
+    (float32 [n, experts]; of equal scores the lower number), weights (float32 [n, top]) their scores."""
+    _gpu(chosen, weights, logits)
+    n, E, ld = _f32rows(logits, "router_topk logits")
+    _check(chosen.dtype == torch.int32 and chosen.is_contiguous() and tuple(chosen.shape) == (n, top), "router_topk: chosen int32 [n, top]")
+    _check(weights.dtype == torch.float32 and weights.is_contiguous() and tuple(weights.shape) == (n, top), "router_topk: weights float32 [n, top]")
+    lib.core().call("hfee_router_topk", _ptr(logits), ld, n, E, int(top), _ptr(chosen), _ptr(weights), _stream())
 
 
 def moe_down(x, act, w_down, top: int, weight: float = 1.0, pair_weights=None, chosen=None, table=None, token_ids=None,
@@ -1320,18 +1478,22 @@ def moe_grouped_fits(dtype, width: int, ff: int) -> bool:
 
 
 def moe_grouped(x, h, w_gate, w_up, w_down, top: int, order, tiles, act, y=None, weight: float = 1.0, pair_weights=None,
-                chosen=None, table=None, token_ids=None):
+                chosen=None, table=None, token_ids=None, in_weights=None):
     """x[t] += sum_j weight_tj * w_down[e_j] @ (silu(w_gate[e_j] @ h[t]) * (w_up[e_j] @ h[t])), bfloat16, with the
     step's (token, expert) pairs grouped by expert on the device and multiplied in tiles on the matrix cores.
     order: int32 [n * top]; tiles: int32 [3 * moe_group_tiles(n, top, experts) + 1]; act: bfloat16
-    [n * top, ff]; y: float32 [n * top, width] (where top > 1): scratch."""
-    _gpu(x, h, w_gate, w_up, w_down, order, tiles, act, y, pair_weights, chosen, table, token_ids)
+    [n * top, ff]; y: float32 [n * top, width] (where top > 1): scratch.  w_gate None: experts without a gate,
+    relu(in_weights[t, j] * (w_up[e_j] @ h[t]))^2 in the gate's place (then without pair_weights)."""
+    _gpu(x, h, w_gate, w_up, w_down, order, tiles, act, y, pair_weights, chosen, table, token_ids, in_weights)
     n, width, ldh = _rows2d(h, "moe_grouped h")
     nx, wx, ldx = _f32rows(x, "moe_grouped x")
-    E, F, W = w_gate.shape
-    _check(nx == n and wx == width == W and w_up.shape == w_gate.shape and tuple(w_down.shape) == (E, width, F)
-           and w_gate.is_contiguous() and w_up.is_contiguous() and w_down.is_contiguous(), "moe_grouped: shapes")
-    _check(h.dtype == w_gate.dtype == w_up.dtype == w_down.dtype == act.dtype == torch.bfloat16, "moe_grouped: bfloat16 operands")
+    E, F, W = w_up.shape
+    _check(nx == n and wx == width == W and tuple(w_down.shape) == (E, width, F) and w_up.is_contiguous() and w_down.is_contiguous()
+           and (w_gate is None or (w_gate.shape == w_up.shape and w_gate.is_contiguous() and w_gate.dtype == torch.bfloat16)),
+           "moe_grouped: shapes")
+    _check(h.dtype == w_up.dtype == w_down.dtype == act.dtype == torch.bfloat16, "moe_grouped: bfloat16 operands")
+    _in_weights(in_weights, w_gate, n, top, "moe_grouped")
+    _check(w_gate is not None or pair_weights is None, "moe_grouped: experts without a gate take their weights on the input")
     _check(act.is_contiguous() and act.numel() >= n * top * F, "moe_grouped: act [n * top, ff]")
     _check(order.dtype == tiles.dtype == torch.int32 and order.is_contiguous() and tiles.is_contiguous()
            and order.numel() >= n * top and tiles.numel() >= 3 * moe_group_tiles(n, top, E) + 1, "moe_grouped: order and tiles")
@@ -1344,4 +1506,4 @@ def moe_grouped(x, h, w_gate, w_up, w_down, top: int, order, tiles, act, y=None,
     _experts_of(chosen, table, token_ids, n, top, "moe_grouped")
     lib.core().call("hfee_moe_grouped", _ptr(x), ldx, _ptr(h), ldh, _ptr(w_gate), _ptr(w_up), _ptr(w_down), _ptr(chosen),
                     _ptr(table), _ptr(token_ids), _ptr(pair_weights), float(weight), top, E, F, width, n, _ptr(order),
-                    _ptr(tiles), _ptr(act), _ptr(y), _stream())
+                    _ptr(tiles), _ptr(act), _ptr(y), _ptr(in_weights), _stream())

@@ -7,7 +7,12 @@ x += mixer(norm(x)); x += feed_forward(norm(x)).
 x += norm_b(mixer(norm_a(x))); x += norm_d(feed_forward(norm_c(x))), with four norms of their own
 weights, and a layer may have no feed-forward.  The sub-layers write float32 rows
 (`forward_into`); one launch norms them, adds them to the stream and makes the norm of the new
-stream for whatever follows (`ops.norm_add`), across layers too.
+stream for whatever follows (`ops.norm_add`), across layers too.  With the parameter `residual_gate`
+every sub-layer's result passes a gate before its norm: y * sigmoid(W_g h + b_g), h the sub-layer's own
+input, W_g [width, width] and b_g a sub-layer; the gate's product runs beside the sub-layer, its sigmoid,
+the multiplication, the norm and the addition are one launch (`ops.gated_norm_add`), which also takes a
+second result with the two scales of a mixer that is two mixers side by side (what its `forward_into`
+returns).
 
 "parallel" has one norm whose output both sub-layers read: with h = norm(x),
 x += mixer(h) + feed_forward(h).  Both add their last product straight into the float32 stream, the
@@ -19,7 +24,9 @@ import torch
 
 from ..config.specs import LayerSpec
 from ..kernels import ops
+from ..weights.spec import TensorSpec
 from .base import LazyNorm, Part, lookup, register_block
+from .kv_attention import product, tiles_of
 
 
 @register_block("prenorm")
@@ -83,10 +90,13 @@ class PreNormBlock(Part):
 @register_block("sandwich")
 class SandwichBlock(Part):
     """Tensor names by role: mixer_norm, mixer_post_norm, feed_forward_norm, feed_forward_post_norm
-    (the whole name behind the layer's prefix), mixer and feed_forward (prefixes)."""
+    (the whole name behind the layer's prefix), mixer and feed_forward (prefixes); with `residual_gate`
+    also mixer_gate, mixer_gate_bias, feed_forward_gate, feed_forward_gate_bias."""
 
     def __init__(self, spec: LayerSpec, dtype: torch.dtype):
         self.spec, self.dtype, self.hidden = spec, dtype, spec.hidden
+        self.gated = bool(spec.get("residual_gate", False))
+        self.gates = {}                  # role -> (weight, tiles, float32 bias), once bound
 
         def norm(norm_spec, role):
             return lookup("norm", norm_spec.kind)(norm_spec, spec.name_of(role, role + ".weight"))
@@ -116,33 +126,72 @@ class SandwichBlock(Part):
     def key_layout(self):
         return getattr(self.mixer, "key_layout", lambda: None)()
 
+    def _gate_roles(self):
+        if not self.gated:
+            return []
+        return ["mixer"] + (["feed_forward"] if self.feed_forward is not None else [])
+
     def tensor_specs(self):
-        return [s for p in self._own() for s in p.tensor_specs()]
+        specs = [s for p in self._own() for s in p.tensor_specs()]
+        for role in self._gate_roles():
+            specs += [TensorSpec(self.spec.name_of(role + "_gate", role + "_gate.weight"), (self.hidden, self.hidden)),
+                      TensorSpec(self.spec.name_of(role + "_gate_bias", role + "_gate.bias"), (self.hidden,), role="vector")]
+        return specs
 
     def bind(self, tensors):
         for p in self._own():
             p.bind(tensors)
+        for role in self._gate_roles():
+            w = tensors.pop(self.spec.name_of(role + "_gate", role + "_gate.weight")).contiguous()
+            b = tensors.pop(self.spec.name_of(role + "_gate_bias", role + "_gate.bias")).to(torch.float32).contiguous()
+            self.gates[role] = (w, tiles_of(self.dtype, w)[0], b)
 
     chains_norms = True
 
     def begin(self, ctx, x):
         return LazyNorm(ctx, self.mixer_norm, x)
 
+    def _gate_of(self, ctx, role, h):
+        """The gate's logits of a sub-layer (engine dtype, before bias and sigmoid), and its bias."""
+        if role not in self.gates:
+            return None, None
+        w, tiles, bias = self.gates[role]
+        logits = ctx.rows("block.gate", self.hidden)
+        product(ctx, logits, h.tensor(), w, tiles)
+        return logits, bias
+
     @staticmethod
     def _rows_of(part, ctx, h, width, *args):
-        """The sub-layer's output as float32 rows (not yet added anywhere)."""
+        """The sub-layer's output as float32 rows (not yet added anywhere), and what `forward_into`
+        returned: None, or dict(y2, scales) of a part whose result is scales[0] * rows + scales[1] * y2."""
         y = ctx.rows("block.sublayer_rows", width, torch.float32)
+        second = None
         if hasattr(part, "forward_into"):
-            part.forward_into(ctx, y, h if part.takes_lazy_norm else h.tensor(), *args)
+            second = part.forward_into(ctx, y, h if part.takes_lazy_norm else h.tensor(), *args)
         else:           # a part that only knows how to add: into rows of zeros
             y.zero_()
             part.forward_add(ctx, y, h if part.takes_lazy_norm else h.tensor(), *args)
-        return y
+        return y, second
 
     @staticmethod
-    def _add_normed(ctx, x, y, post_norm, bias, following):
+    def _add_normed(ctx, x, y, post_norm, bias, following, second=None, gate=None, gate_bias=None):
         """x += post_norm(y + bias), and the norm that follows in the same launch where it is of the
-        same form and nobody has made it yet."""
+        same form and nobody has made it yet.  second / gate: see `ops.gated_norm_add`."""
+        if second is not None or gate is not None:
+            if bias is not None:
+                raise ValueError("a gated sub-layer has no bias behind its last product")
+            weight, eps = post_norm.fused_form_f32()
+            more = dict(y2=second["y2"], scales=second["scales"]) if second is not None else {}
+            nxt = following.fusable() if following is not None else None
+            if nxt is not None and following._tensor is None and following.pending is None:
+                out = ctx.rows("block.normed", x.shape[1])
+                w2, eps2 = following.norm.fused_form_f32()
+                ops.gated_norm_add(x, y, weight, eps, gate=gate, gate_bias=gate_bias, next_out=out, next_weight=w2,
+                                   next_eps=eps2, **more)
+                following._tensor = out
+            else:
+                ops.gated_norm_add(x, y, weight, eps, gate=gate, gate_bias=gate_bias, **more)
+            return
         weight, eps = post_norm.fused_form()
         nxt = following.fusable() if following is not None else None
         if nxt is not None and following._tensor is None and following.pending is None and nxt[0].dtype == weight.dtype:
@@ -154,14 +203,17 @@ class SandwichBlock(Part):
 
     def forward(self, ctx, x, entry, h_in=None, h_next=None):
         h = h_in if h_in is not None else self.begin(ctx, x)
-        y = self._rows_of(self.mixer, ctx, h, self.hidden, entry.cache, entry.writes_cache)
+        gate, gate_bias = self._gate_of(ctx, "mixer", h)
+        y, second = self._rows_of(self.mixer, ctx, h, self.hidden, entry.cache, entry.writes_cache)
         if self.feed_forward is None:
-            self._add_normed(ctx, x, y, self.mixer_post_norm, getattr(self.mixer, "output_bias", None), h_next)
+            self._add_normed(ctx, x, y, self.mixer_post_norm, getattr(self.mixer, "output_bias", None), h_next, second, gate, gate_bias)
             return
         h2 = LazyNorm(ctx, self.feed_forward_norm, x)
-        self._add_normed(ctx, x, y, self.mixer_post_norm, getattr(self.mixer, "output_bias", None), h2)
-        y = self._rows_of(self.feed_forward, ctx, h2, self.hidden)
-        self._add_normed(ctx, x, y, self.feed_forward_post_norm, getattr(self.feed_forward, "output_bias", None), h_next)
+        self._add_normed(ctx, x, y, self.mixer_post_norm, getattr(self.mixer, "output_bias", None), h2, second, gate, gate_bias)
+        gate, gate_bias = self._gate_of(ctx, "feed_forward", h2)
+        y, second = self._rows_of(self.feed_forward, ctx, h2, self.hidden)
+        self._add_normed(ctx, x, y, self.feed_forward_post_norm, getattr(self.feed_forward, "output_bias", None), h_next,
+                         second, gate, gate_bias)
 
 
 @register_block("parallel")

@@ -2,7 +2,9 @@
 
 Embedding: a row gather into the float32 residual stream, no scaling
 (/root/reference/internal/llm/forward.go:75-77) unless the spec gives a `scale`, by which every
-element is multiplied in float32 on its way.  Head: final norm and the
+element is multiplied in float32 on its way; with `position_table` (a tensor name) and `positions` (its
+rows) a learned vector a position is added to the row, table[p] for a token at position p of its
+sequence, in float32 and not scaled.  Head: final norm and the
 vocabulary product only for the rows whose logits are wanted
 (/root/reference/internal/llm/forward.go:117-141); it shares the embedding table
 when the model has no separate head (/root/reference/internal/llm/model.go:118-121).
@@ -27,12 +29,26 @@ class Embedding(Part):
         self.name, self.vocab, self.hidden = name, vocab, hidden
         self.scale = float(spec.get("scale", 1.0))
         self.table = None
+        self.position_name, self.positions = spec.get("position_table"), int(spec.get("positions", 0) or 0)
+        self.position_table = None
+        if self.position_name is not None and self.positions < 1:
+            raise ValueError("an embedding with learned positions needs the number of positions")
 
     def tensor_specs(self):
-        return [TensorSpec(self.name, (self.vocab, self.hidden))]
+        specs = [TensorSpec(self.name, (self.vocab, self.hidden))]
+        if self.position_name is not None:
+            specs.append(TensorSpec(self.position_name, (self.positions, self.hidden)))
+        return specs
 
     def bind(self, tensors):
         self.table = tensors[self.name].contiguous()
+        if self.position_name is not None:
+            self.position_table = tensors[self.position_name].contiguous()
+
+    def prepare(self, info):
+        if self.position_table is not None and info.num_positions > self.positions:
+            raise ValueError(f"the model has learned vectors for {self.positions} positions, the engine was made for "
+                             f"{info.num_positions}")
 
     # forward takes the normed input of the first block as `then` (a LazyNorm), and may do
     # the first half of that norm on its way
@@ -40,9 +56,11 @@ class Embedding(Part):
 
     def forward(self, ctx, x, then=None):
         emit = None
-        if then is not None and self.scale == 1.0 and ops.can_embed_emit(self.table, ctx.n):
+        if then is not None and self.scale == 1.0 and self.position_table is None and ops.can_embed_emit(self.table, ctx.n):
             emit = then.offer(blocks=ops.embed_emit_blocks(self.hidden))
         ops.embed(x, self.table, ctx.token_ids, emit=emit, scale=self.scale)
+        if self.position_table is not None:
+            ops.add_table_rows(x, self.position_table, ctx.positions)
 
 
 @register_head("norm_linear")

@@ -1,4 +1,4 @@
-"""Two mixers over one family of attention kernels, whose keys and values have sizes of their own.
+"""Three mixers over one family of attention kernels, whose keys and values have sizes of their own.
 
 "kv_attention": grouped attention.  H query heads over G key/value heads (query head h reads
 key/value head h // (H/G)), key size Dk, value size Dv; q and k are rotated in the first
@@ -19,7 +19,14 @@ size rank + rotated dims), the weighted sum is taken over the latents themselves
 rank), and W_uv,h is applied to the result.  Prompt portions and single tokens then run the same
 kernels, and a token's logits do not depend on how its prompt was cut.
 
-Both write float32 rows for a block that norms a sub-layer's output before it adds it to the
+"sigmoid_attention": grouped attention without a softmax and without a rotation.  q and k are divided
+by their root mean square over each head (eps `norm_eps`) and multiplied by a weight of the head's size
+that all heads share, one for q and one for k; with `temperature` = (coef, every) the query at position p
+is also multiplied by 1 + coef * ln(floor((p + 1) / every) + 1); score = q.k * scale; a key up to the
+token's own position weighs sigmoid(score + b_h), b_h a learned number a head, and the weights are not
+normalized over the keys: every key adds on its own, however far back it lies.
+
+All write float32 rows for a block that norms a sub-layer's output before it adds it to the
 residual stream (`forward_into`); `forward_add` is there for the other blocks.
 
 In bfloat16 with sizes that are multiples of 16 the matrix-core kernels run (rows of a prompt
@@ -57,15 +64,17 @@ def plan_items(plan, rows: int) -> None:
         plan.host["attention_kv.single_max_position"] = max([p for _, _, p, _ in singles], default=0)
 
 
-def attend(ctx, out, q, cache, tables, num_heads, kv_heads, dk, dv, scale, sinks, matrix: bool) -> None:
+def attend(ctx, out, q, cache, tables, num_heads, kv_heads, dk, dv, scale, sinks, matrix: bool, weights: str = "softmax") -> None:
+    """weights "sigmoid": no softmax, `sinks` holds the number a head that joins every score."""
     if not matrix:
         ops.attention_kv_plain(out, q, cache, ctx.positions, ctx.token_segment, tables, num_heads, kv_heads, dk, dv,
-                               ctx.page_size, scale, sinks)
+                               ctx.page_size, scale, sinks, weights=weights)
         return
-    portions = ctx.extra[f"attention_kv.portions.{ops.attention_kv_rows(dk, dv, num_heads // kv_heads)}"]
+    portions = ctx.extra[f"attention_kv.portions.{ops.attention_kv_rows(dk, dv, num_heads // kv_heads, weights)}"]
     singles = ctx.extra["attention_kv.singles"]
     if portions.shape[0]:
-        ops.attention_kv_bf16(out, q, cache, portions, 0, tables, num_heads, kv_heads, dk, dv, ctx.page_size, scale, sinks)
+        ops.attention_kv_bf16(out, q, cache, portions, 0, tables, num_heads, kv_heads, dk, dv, ctx.page_size, scale, sinks,
+                              weights=weights)
     count = singles.shape[0]
     if count:
         # under a captured graph the split count is fixed for the whole width of the block table
@@ -78,7 +87,7 @@ def attend(ctx, out, q, cache, tables, num_heads, kv_heads, dk, dv, scale, sinks
             partial = ctx.workspace.flat("attention_kv.partial", ops.attention_kv_partial_words(count, num_heads, dv, splits),
                                          torch.float32)
         ops.attention_kv_bf16(out, q, cache, singles, 1, tables, num_heads, kv_heads, dk, dv, ctx.page_size, scale, sinks,
-                              partial=partial, splits=splits)
+                              partial=partial, splits=splits, weights=weights)
 
 
 def tiles_of(dtype, *weights):
@@ -104,6 +113,7 @@ def product(ctx, out, x, weight, tiles=None, add: bool = False) -> None:
 
 class _KvMixer(Mixer):
     graph_safe = True
+    weights = "softmax"       # how a key's weight comes from its score (`ops.KEY_WEIGHTS`)
 
     def _names(self, spec, defaults):
         given = dict(spec.get("names") or ())
@@ -119,7 +129,7 @@ class _KvMixer(Mixer):
 
     def plan(self, plan):
         if self.matrix:
-            plan_items(plan, ops.attention_kv_rows(*self.kernel_sizes))
+            plan_items(plan, ops.attention_kv_rows(*self.kernel_sizes, self.weights))
 
     def forward_add(self, ctx, x, h, cache_layer: int, writes_cache: bool):
         y = ctx.rows("mixer.rows_out", self.hidden, torch.float32)
@@ -207,6 +217,77 @@ class KvAttention(_KvMixer):
                      v_mix=self.blend_weight)
         att = ctx.rows("kv_attention.out", self.out_width)
         attend(ctx, att, q, cache, tables, H, G, dk, dv, self.scale, self.sinks, self.matrix)
+        product(ctx, out, att, self.w_o, self.w_o_tiles)
+
+
+@register_mixer("sigmoid_attention")
+class SigmoidAttention(_KvMixer):
+    """Tensor names by role: q, k, v, o (matrices), q_norm, k_norm ([key_dim]), head_bias ([heads])."""
+    weights = "sigmoid"
+
+    def __init__(self, spec: MixerSpec, prefix: str, dtype: torch.dtype):
+        self.prefix, self.dtype = prefix, dtype
+        self.hidden = spec.get("hidden")
+        self.num_heads = spec.get("num_heads")
+        self.kv_heads = spec.get("num_kv_heads", self.num_heads)
+        self.dk = spec.get("key_dim")
+        self.dv = spec.get("value_dim", self.dk)
+        self.scale = float(spec.get("scale", self.dk ** -0.5))
+        self.norm_eps = float(spec.get("norm_eps", 1e-6))
+        self.temperature = spec.get("temperature")          # None | (coef, every)
+        if self.num_heads % self.kv_heads:
+            raise ValueError(f"{self.num_heads} heads are not a multiple of {self.kv_heads} kv heads")
+        if self.temperature is not None and int(self.temperature[1]) < 1:
+            raise ValueError("the query temperature grows in steps of at least one position")
+        self.position = None
+        self.names = self._names(spec, dict(q="q_proj.weight", k="k_proj.weight", v="v_proj.weight", o="o_proj.weight",
+                                            q_norm="q_norm.weight", k_norm="k_norm.weight", head_bias="head_bias"))
+        self.q_width, self.k_width, self.v_width = self.num_heads * self.dk, self.kv_heads * self.dk, self.kv_heads * self.dv
+        self.out_width = self.num_heads * self.dv
+        self.kernel_sizes = (self.dk, self.dv, self.num_heads // self.kv_heads)
+        self.matrix = self._matrix(self.dk, self.dv, self.q_width + self.k_width + self.v_width, self.out_width)
+
+    def tensor_specs(self):
+        n = self.names
+        return [TensorSpec(n["q"], (self.q_width, self.hidden)), TensorSpec(n["k"], (self.k_width, self.hidden)),
+                TensorSpec(n["v"], (self.v_width, self.hidden)), TensorSpec(n["o"], (self.hidden, self.out_width)),
+                TensorSpec(n["q_norm"], (self.dk,), role="vector", init=("one_plus_normal",)),
+                TensorSpec(n["k_norm"], (self.dk,), role="vector", init=("one_plus_normal",)),
+                TensorSpec(n["head_bias"], (self.num_heads,), role="vector")]
+
+    def bind(self, tensors):
+        n = self.names
+        self.w_qkv = torch.cat([tensors.pop(n["q"]), tensors.pop(n["k"]), tensors.pop(n["v"])], dim=0).contiguous()
+        self.w_o = tensors.pop(n["o"]).contiguous()
+        self.q_norm = tensors.pop(n["q_norm"]).to(torch.float32).contiguous()
+        self.k_norm = tensors.pop(n["k_norm"]).to(torch.float32).contiguous()
+        self.head_bias = tensors.pop(n["head_bias"]).to(torch.float32).contiguous()
+        self.w_qkv_tiles, self.w_o_tiles = tiles_of(self.dtype, self.w_qkv, self.w_o)
+
+    def cache_spec(self):
+        return CacheNeed("full", (self.kv_heads, self.dk + self.dv), 0, layout=_LAYOUT)
+
+    def key_layout(self):
+        return (self.kv_heads, self.dk, self.dv, "normed", self.norm_eps)
+
+    def forward_into(self, ctx, out, h, cache_layer: int, writes_cache: bool):
+        hn = h.tensor() if isinstance(h, LazyNorm) else h
+        H, G, dk, dv = self.num_heads, self.kv_heads, self.dk, self.dv
+        cache = ctx.storage.layer(cache_layer, (G, ctx.page_size * (dk + dv)))
+        tables = self._tables(ctx, cache_layer)
+        qkv = ctx.rows("kv_attention.qkv", self.q_width + self.k_width + self.v_width)
+        q = qkv[:, :self.q_width]
+        k = v = None
+        if writes_cache:
+            product(ctx, qkv, hn, self.w_qkv, self.w_qkv_tiles)
+            k = qkv[:, self.q_width:self.q_width + self.k_width]
+            v = qkv[:, self.q_width + self.k_width:]
+        else:       # this run of the layer reads keys and values that another run wrote
+            ops.linear(q, hn, self.w_qkv[:self.q_width])
+        ops.qk_norm_write(q, k, v, ctx.positions, ctx.token_segment, tables, cache, self.q_norm, self.k_norm, self.norm_eps,
+                          H, G, dk, dv, ctx.page_size, temperature=self.temperature)
+        att = ctx.rows("kv_attention.out", self.out_width)
+        attend(ctx, att, q, cache, tables, H, G, dk, dv, self.scale, self.head_bias, self.matrix, weights="sigmoid")
         product(ctx, out, att, self.w_o, self.w_o_tiles)
 
 

@@ -1,4 +1,4 @@
-"""A feed-forward of many small gated experts, of which every token uses `top`.
+"""Feed-forwards of many small experts, of which every token uses `top`.
 
 "table_moe": no router.  A table [vocabulary, top] of integers gives every token id its experts (the
 entries of a row differ); each counts 1 / top.  Expert: down(act(gate(h)) * up(h)), act the SiLU, no
@@ -8,6 +8,13 @@ runs on the device from the step's token ids, so a step may be replayed from a r
 with more (token, expert) pairs than experts groups the pairs by expert on the device and multiplies them
 in tiles on the matrix cores (bfloat16, sizes that are multiples of 32); a step of few tokens, and
 float32, reads each token's experts row by row.
+
+"routed_moe": a router chooses.  z = W_router h in float32; scores s = sigmoid(z); the `top` experts with
+the largest scores are a token's, and their weights are those scores as they are (not renormalized).
+Expert: down(relu(up(w h))^2), no gate and no biases: the weight w multiplies the expert's input (it joins
+the up product's float32 sum, which is the same product).  The output is the sum of the chosen experts'
+outputs.  It writes float32 rows (`forward_into`) for a block that norms them, or adds them to the stream.
+Steps of many tokens go through the same grouped kernels as above, few tokens and float32 row by row.
 """
 from __future__ import annotations
 
@@ -78,3 +85,79 @@ class TableMoE(FeedForward):
         act = ctx.rows("table_moe.act", self.top * self.intermediate).view(ctx.n * self.top, self.intermediate)
         ops.moe_up(act, hn, self.w_gate, self.w_up, self.top, table=self.table, token_ids=ctx.token_ids)
         ops.moe_down(x, act, self.w_down, self.top, weight=1.0 / self.top, table=self.table, token_ids=ctx.token_ids)
+
+
+@register_feed_forward("routed_moe")
+class RoutedMoE(FeedForward):
+    """Tensor names by role: router ([experts, hidden]); expert (a format for the expert's number), up, down."""
+    graph_safe = True
+
+    def __init__(self, spec: FeedForwardSpec, prefix: str, dtype: torch.dtype):
+        self.prefix, self.dtype = prefix, dtype
+        self.hidden = spec.get("hidden")
+        self.intermediate = spec.get("intermediate")
+        self.experts, self.top = spec.get("experts"), spec.get("top")
+        if spec.get("activation", "relu2") != "relu2" or spec.get("score", "sigmoid") != "sigmoid":
+            raise ValueError("the routed experts' activation is the square of relu, their scores are sigmoids")
+        if spec.get("weight_on", "input") != "input" or spec.get("renormalize", False):
+            raise ValueError("the routed experts' weights multiply their inputs and are not renormalized")
+        if not 1 <= self.top <= self.experts:
+            raise ValueError(f"a token uses 1 to {self.experts} experts, not {self.top}")
+        given = dict(spec.get("names") or ())
+        self.expert_names = given.get("expert", "experts.{}.")
+        self.roles = {r: given.get(r, d) for r, d in dict(up="up_proj.weight", down="down_proj.weight",
+                                                         router="router.weight").items()}
+        self.output_bias = None
+
+    def _name(self, e: int, role: str) -> str:
+        return self.prefix + self.expert_names.format(e) + self.roles[role]
+
+    def tensor_specs(self):
+        specs = []
+        for e in range(self.experts):
+            specs += [TensorSpec(self._name(e, "up"), (self.intermediate, self.hidden)),
+                      TensorSpec(self._name(e, "down"), (self.hidden, self.intermediate))]
+        specs.append(TensorSpec(self.prefix + self.roles["router"], (self.experts, self.hidden)))
+        return specs
+
+    def bind(self, tensors):
+        E = range(self.experts)
+        self.w_up = torch.stack([tensors.pop(self._name(e, "up")) for e in E]).contiguous()
+        self.w_down = torch.stack([tensors.pop(self._name(e, "down")) for e in E]).contiguous()
+        self.w_router = tensors.pop(self.prefix + self.roles["router"]).contiguous()
+
+    def _choose(self, ctx, hn):
+        n, top = ctx.n, self.top
+        logits = ctx.rows("routed_moe.logits", self.experts, torch.float32)
+        ops.linear(logits, hn, self.w_router)
+        ws = ctx.workspace
+        chosen = ws.flat("routed_moe.chosen", ws.capacity * top, torch.int32)[:n * top].view(n, top)
+        weights = ws.flat("routed_moe.weights", ws.capacity * top, torch.float32)[:n * top].view(n, top)
+        ops.router_topk(chosen, weights, logits, top)
+        return chosen, weights
+
+    def _run(self, ctx, out, h, add: bool):
+        hn = h.tensor() if isinstance(h, LazyNorm) else h
+        n, top = ctx.n, self.top
+        chosen, weights = self._choose(ctx, hn)
+        if n * top > self.experts and ops.moe_grouped_fits(self.dtype, self.hidden, self.intermediate) \
+                and hn.data_ptr() % 16 == 0 and hn.stride(0) % 8 == 0:
+            ws = ctx.workspace
+            order = ws.flat("table_moe.order", ws.capacity * top, torch.int32)
+            tiles = ws.flat("table_moe.tiles", 3 * ops.moe_group_tiles(ws.capacity, top, self.experts) + 1, torch.int32)
+            act = ctx.rows("table_moe.act", top * self.intermediate)
+            y = ctx.rows("table_moe.rows", top * self.hidden, torch.float32) if top > 1 else None
+            if not add:
+                out.zero_()
+            ops.moe_grouped(out, hn, None, self.w_up, self.w_down, top, order, tiles, act, y, weight=1.0, chosen=chosen,
+                            in_weights=weights)
+            return
+        act = ctx.rows("table_moe.act", top * self.intermediate).view(n * top, self.intermediate)
+        ops.moe_up(act, hn, None, self.w_up, top, chosen=chosen, in_weights=weights)
+        ops.moe_down(out, act, self.w_down, top, weight=1.0, chosen=chosen, accumulate=add)
+
+    def forward_into(self, ctx, out, h):
+        self._run(ctx, out, h, add=False)
+
+    def forward_add(self, ctx, x, h):
+        self._run(ctx, x, h, add=True)

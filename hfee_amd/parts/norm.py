@@ -35,6 +35,14 @@ class RMSNorm(Norm):
     def fused_form(self):
         return self.weight, self.eps
 
+    def fused_form_f32(self):
+        """(weight as float32, eps), for the launches that take their weights in float32 only."""
+        if self.weight.dtype == torch.float32:
+            return self.weight, self.eps
+        if getattr(self, "_weight_f32", None) is None:
+            self._weight_f32 = self.weight.to(torch.float32).contiguous()
+        return self._weight_f32, self.eps
+
     def forward(self, ctx, out, x, rows=None):
         ops.rmsnorm(out, x, self.weight, self.eps, rows)
 

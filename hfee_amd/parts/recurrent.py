@@ -1,9 +1,10 @@
-"""Mixers that keep a matrix of fixed size for every request instead of a growing cache.
+"""Mixers that keep a state of fixed size for every request instead of a growing cache.
 
-Both hold, for each head, S [dim, vdim] in float32 in the request's state slot (zero when the request
-is admitted), walk a step's tokens of a request in order from it, and leave the new state there; a
-decay acts on the rows of S, one number a key channel.  What enters the recurrence besides the
-projections themselves is made in float32: decays, step sizes, writing strengths, unit norms.
+"gated_delta", "gla" and "state_space" hold, for each head, S [dim, vdim] in float32 in the request's
+state slot (zero when the request is admitted), walk a step's tokens of a request in order from it, and
+leave the new state there; a decay acts on the rows of S, one number a key channel (a head in
+"state_space").  "rglru" holds one number a channel.  What enters a recurrence besides the projections
+and short convolutions themselves is made in float32: decays, step sizes, writing strengths, gates, unit norms.
 
 "gated_delta": q, k (`num_qk_heads` heads of `dim`; head h reads q/k head h // (heads / qk heads)) and v
 (`num_heads` heads of `vdim`) each pass a short causal convolution per channel (`conv` taps, no bias,
@@ -17,10 +18,25 @@ sigmoid(W_g2 W_g1 h); then the output product.
 "gla": q = W_q h dim^(-1/2), k, v; a = sigmoid(W_a2 W_a1 h + bias)^(1/tau);
 S <- diag(a) S + k v^T; o = S^T q; each head's o normed as above with a weight shared by the heads,
 the heads side by side times silu(W_g h); then the output product.
+
+"state_space" (state-space duality): one product gives [z | x | B | C | dt] (z, x: `num_heads` heads of
+`vdim`; B, C: `groups` groups of `state`; dt a head).  x, B and C together pass a short causal convolution
+per channel with a bias and a SiLU.  dt = softplus(dt + dt_bias); per head (head h reads group
+h // (heads / groups)), with a = exp(-exp(A_h) dt): S <- a S + dt B x^T (S [state, vdim]),
+y = S^T C + D_h x.  The heads side by side are multiplied by silu(z) and then divided by their root mean
+square in `norm_groups` equal parts (eps `norm_eps`), times a weight an element; then the output product.
+
+"rglru" (a real-gated linear recurrent unit between two branches of `width` channels): y =
+gelu_tanh(W_y h + b_y); u = conv(W_x h + b_x), a short causal convolution per channel with a bias and no
+activation.  u is cut into `blocks` equal parts; in part b, r = sigmoid(R_b u_b + c_b) and
+i = sigmoid(I_b u_b + d_b) with square matrices R_b, I_b, in float32.  With a = exp(-decay_scale * r *
+softplus(lam)), lam a number a channel: S <- a S + sqrt(1 - a^2) * i * u; the output product reads S * y.
 """
 from __future__ import annotations
 
 import torch
+
+import torch.nn.functional as F
 
 from ..config.specs import MixerSpec
 from ..kernels import ops
@@ -194,3 +210,160 @@ class GatedLinearAttention(_StateMixer):
         gated = ctx.rows("gla.out", self.v_width)
         ops.head_norm_gate(gated, o, proj[:, self.at_g:self.at_a], self.norm_weight, H, V, self.norm_eps, "silu")
         product(ctx, x, gated, self.w_o, self.w_o_tiles, add=True)
+
+
+@register_mixer("state_space")
+class StateSpace(_StateMixer):
+    """Tensor names by role: in ([z | x | B | C | dt] rows), conv ([channels, taps]), conv_bias, dt_bias,
+    a_log, skip ([heads]), norm ([inner]), o."""
+
+    def __init__(self, spec: MixerSpec, prefix: str, dtype: torch.dtype):
+        self.prefix, self.dtype = prefix, dtype
+        self.hidden = spec.get("hidden")
+        self.heads, self.vdim = spec.get("num_heads"), spec.get("vdim")
+        self.state_size, self.groups = spec.get("state"), spec.get("groups", 1)
+        self.taps = spec.get("conv")
+        self.norm_groups = spec.get("norm_groups", 1)
+        self.norm_eps = float(spec.get("norm_eps", 1e-6))
+        self.inner = self.heads * self.vdim
+        if self.heads % self.groups:
+            raise ValueError(f"{self.heads} heads are not a multiple of {self.groups} groups")
+        if self.inner % self.norm_groups:
+            raise ValueError(f"{self.inner} values are not {self.norm_groups} equal parts")
+        if self.taps < 1:
+            raise ValueError("the short convolution has at least one tap")
+        self.names = self._names(spec, dict(
+            **{"in": "in_proj.weight"}, conv="conv.weight", conv_bias="conv.bias", dt_bias="dt_bias", a_log="A_log",
+            skip="D", norm="norm.weight", o="out_proj.weight"))
+        self.bc_width = self.groups * self.state_size
+        self.channels = self.inner + 2 * self.bc_width
+        self.in_width = 2 * self.inner + 2 * self.bc_width + self.heads
+
+    def tensor_specs(self):
+        n = self.names
+        return [TensorSpec(n["in"], (self.in_width, self.hidden)),
+                TensorSpec(n["conv"], (self.channels, self.taps), role="vector"),
+                TensorSpec(n["conv_bias"], (self.channels,), role="vector"),
+                TensorSpec(n["dt_bias"], (self.heads,), role="vector"), TensorSpec(n["a_log"], (self.heads,), role="vector"),
+                TensorSpec(n["skip"], (self.heads,), role="vector", init=("one_plus_normal",)),
+                TensorSpec(n["norm"], (self.inner,), role="vector", init=("one_plus_normal",)),
+                TensorSpec(n["o"], (self.hidden, self.inner))]
+
+    def bind(self, tensors):
+        n = self.names
+        f32 = lambda name: tensors.pop(name).to(torch.float32).contiguous()      # noqa: E731
+        self.w_in, self.w_o = tensors.pop(n["in"]).contiguous(), tensors.pop(n["o"]).contiguous()
+        self.conv_taps, self.conv_bias = f32(n["conv"]), f32(n["conv_bias"])
+        self.dt_bias, self.a_log, self.skip, self.norm_weight = f32(n["dt_bias"]), f32(n["a_log"]), f32(n["skip"]), f32(n["norm"])
+        self.w_in_tiles, self.w_o_tiles = tiles_of(self.dtype, self.w_in, self.w_o)
+
+    def state_specs(self):
+        return [(self.prefix + "state", (self.heads, *ops.scan_state_shape(self.state_size, self.vdim)), torch.float32),
+                (self.prefix + "conv_state", (self.taps - 1, self.channels), self.dtype)]
+
+    def prepare(self, info):
+        self.state = info.storage.states[self.prefix + "state"]
+        self.conv_state = info.storage.states[self.prefix + "conv_state"]
+
+    def forward_into(self, ctx, out, h, cache_layer: int, writes_cache: bool):
+        hn = h.tensor() if isinstance(h, LazyNorm) else h
+        H, G, N, V, inner = self.heads, self.groups, self.state_size, self.vdim, self.inner
+        rows, lengths, slots = self._segments(ctx)
+        proj = ctx.rows("state_space.in", (self.in_width + 7) // 8 * 8)[:, :self.in_width]
+        product(ctx, proj, hn, self.w_in, self.w_in_tiles)
+        z, raw, dt_raw = proj[:, :inner], proj[:, inner:inner + self.channels], proj[:, inner + self.channels:]
+        conv = ctx.rows("state_space.conv", self.channels, torch.float32)
+        ops.short_conv_silu(conv, raw, self.conv_state, self.conv_taps, ctx.token_segment, rows, slots, out_bias=self.conv_bias)
+        ops.short_conv_keep(self.conv_state, raw, rows, lengths, slots)
+        xs, B, C = conv[:, :inner], conv[:, inner:inner + self.bc_width], conv[:, inner + self.bc_width:]
+        steps = ctx.rows("state_space.steps", 2 * H, torch.float32)
+        dt, decay = steps[:, :H], steps[:, H:]
+        ops.scan_gate(dt, dt_raw, "softplus", bias=self.dt_bias)
+        ops.scan_gate(decay, dt_raw, "step_decay", bias=self.dt_bias, per_head=self.a_log, head_width=1)
+        o = ctx.rows("state_space.read", inner, torch.float32)
+        ops.linear_scan(o, self.state, C, B, xs, decay, dt, rows, lengths, slots, H, G, N, V, "scaled_add", decay_per_head=True)
+        gated = ctx.rows("state_space.out", inner)
+        ops.gate_group_norm(gated, o, xs, self.skip, z, self.norm_weight, H, self.norm_groups, self.norm_eps)
+        product(ctx, out, gated, self.w_o, self.w_o_tiles)
+
+    def forward_add(self, ctx, x, h, cache_layer: int, writes_cache: bool):
+        y = ctx.rows("mixer.rows_out", self.hidden, torch.float32)
+        self.forward_into(ctx, y, h, cache_layer, writes_cache)
+        ops.residual_add(x, y)
+
+
+@register_mixer("rglru")
+class RealGatedRecurrentUnit(_StateMixer):
+    """Tensor names by role: y, y_bias, x, x_bias (the two branches), conv ([width, taps]), conv_bias,
+    decay_gate and input_gate ([blocks, block, block], [out, in]) with decay_gate_bias and input_gate_bias
+    ([blocks, block]), lam ([width]), o."""
+
+    def __init__(self, spec: MixerSpec, prefix: str, dtype: torch.dtype):
+        self.prefix, self.dtype = prefix, dtype
+        self.hidden = spec.get("hidden")
+        self.width, self.blocks = spec.get("width"), spec.get("blocks", 1)
+        self.taps = spec.get("conv")
+        self.decay_scale = float(spec.get("decay_scale", 8.0))
+        if self.width % self.blocks:
+            raise ValueError(f"{self.width} channels are not {self.blocks} equal blocks")
+        if self.taps < 1:
+            raise ValueError("the short convolution has at least one tap")
+        self.block = self.width // self.blocks
+        self.names = self._names(spec, dict(
+            y="y_proj.weight", y_bias="y_proj.bias", x="x_proj.weight", x_bias="x_proj.bias", conv="conv.weight",
+            conv_bias="conv.bias", decay_gate="a_gate.weight", decay_gate_bias="a_gate.bias", input_gate="i_gate.weight",
+            input_gate_bias="i_gate.bias", lam="lambda", o="out_proj.weight"))
+
+    def tensor_specs(self):
+        n, W, nb, bs = self.names, self.width, self.blocks, self.block
+        return [TensorSpec(n["y"], (W, self.hidden)), TensorSpec(n["y_bias"], (W,), role="vector"),
+                TensorSpec(n["x"], (W, self.hidden)), TensorSpec(n["x_bias"], (W,), role="vector"),
+                TensorSpec(n["conv"], (W, self.taps), role="vector"), TensorSpec(n["conv_bias"], (W,), role="vector"),
+                TensorSpec(n["decay_gate"], (nb, bs, bs), role="vector"), TensorSpec(n["decay_gate_bias"], (nb, bs), role="vector"),
+                TensorSpec(n["input_gate"], (nb, bs, bs), role="vector"), TensorSpec(n["input_gate_bias"], (nb, bs), role="vector"),
+                TensorSpec(n["lam"], (W,), role="vector"), TensorSpec(n["o"], (self.hidden, W))]
+
+    def bind(self, tensors):
+        n = self.names
+        f32 = lambda name: tensors.pop(name).to(torch.float32).contiguous()      # noqa: E731
+        # one product for both branches: [y | x]
+        self.w_in = torch.cat([tensors.pop(n["y"]), tensors.pop(n["x"])], dim=0).contiguous()
+        self.w_o = tensors.pop(n["o"]).contiguous()
+        self.y_bias, self.x_bias = f32(n["y_bias"]), f32(n["x_bias"])
+        self.conv_taps, self.conv_bias = f32(n["conv"]), f32(n["conv_bias"])
+        # both gates of a block as one float32 product, [block][in][decay gate's outputs | input gate's outputs]
+        gates = torch.cat([f32(n["decay_gate"]), f32(n["input_gate"])], dim=1)          # [blocks, 2 block (out), block (in)]
+        self.w_gates = gates.transpose(1, 2).contiguous()
+        self.gate_bias = torch.cat([f32(n["decay_gate_bias"]), f32(n["input_gate_bias"])], dim=1).contiguous().view(-1)
+        self.rate = (-self.decay_scale * F.softplus(f32(n["lam"]))).contiguous()       # the decay's logarithm a unit of its gate
+        self.w_in_tiles, self.w_o_tiles = tiles_of(self.dtype, self.w_in, self.w_o)
+
+    def state_specs(self):
+        return [(self.prefix + "state", (self.width,), torch.float32),
+                (self.prefix + "conv_state", (self.taps - 1, self.width), self.dtype)]
+
+    def prepare(self, info):
+        self.state = info.storage.states[self.prefix + "state"]
+        self.conv_state = info.storage.states[self.prefix + "conv_state"]
+
+    def forward_into(self, ctx, out, h, cache_layer: int, writes_cache: bool):
+        hn = h.tensor() if isinstance(h, LazyNorm) else h
+        W = self.width
+        rows, lengths, slots = self._segments(ctx)
+        proj = ctx.rows("rglru.in", 2 * W)
+        product(ctx, proj, hn, self.w_in, self.w_in_tiles)
+        y, raw = proj[:, :W], proj[:, W:]
+        u = ctx.rows("rglru.conv", W, torch.float32)
+        ops.short_conv_silu(u, raw, self.conv_state, self.conv_taps, ctx.token_segment, rows, slots, in_bias=self.x_bias,
+                            out_bias=self.conv_bias, activation="none")
+        ops.short_conv_keep(self.conv_state, raw, rows, lengths, slots, in_bias=self.x_bias)
+        gates = ctx.rows("rglru.gates", 2 * W, torch.float32)
+        ops.head_linear(gates, u, self.w_gates, self.blocks, self.block, 2 * self.block)
+        read = ctx.rows("rglru.read", W)
+        ops.rglru_scan(read, self.state, gates, self.gate_bias, u, self.rate, y, self.y_bias, rows, lengths, slots, self.block)
+        product(ctx, out, read, self.w_o, self.w_o_tiles)
+
+    def forward_add(self, ctx, x, h, cache_layer: int, writes_cache: bool):
+        y = ctx.rows("mixer.rows_out", self.hidden, torch.float32)
+        self.forward_into(ctx, y, h, cache_layer, writes_cache)
+        ops.residual_add(x, y)
