@@ -67,6 +67,16 @@ SABEZEN_SIZES = {
     "4096-wide": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=21504, llama_ff=14336, expert_ff=2048),
 }
 
+# The Ronavik design at the same two layer sizes, beside Sabezen (the closest of the other designs: attention,
+# per-request states and experts): its layers go in turn through a pair of attention without a softmax (heads
+# and head size of the Llama layer of that width) beside a real-gated recurrent unit as wide as the model in
+# blocks of 256 channels, and a state-space mixer (heads of 64 values that make twice the model's width, states
+# of 128, eight groups); every layer has sixteen routed experts without a gate, two a token.
+RONAVIK_SIZES = {
+    "2048-wide": dict(width=2048, heads=16, kv_heads=4, dim=128, expert_ff=1024),
+    "4096-wide": dict(width=4096, heads=32, kv_heads=8, dim=128, expert_ff=2048),
+}
+
 
 CONTEXT = 8192
 PROMPT = 1024
@@ -118,6 +128,13 @@ def parse(argv=None):
                     help="with --sabezen: only this layer size")
     ap.add_argument("--sabezen-design", choices=["both", "sabezen", "llama"], default="both",
                     help="with --sabezen: only one of the two designs (for profiling)")
+    ap.add_argument("--ronavik", action="store_true",
+                    help="the Ronavik design beside the Sabezen design at two layer sizes that resemble real models' "
+                    "layers (random weights): prefill and decode throughput; prints its own JSON line")
+    ap.add_argument("--ronavik-size", choices=sorted(RONAVIK_SIZES), default=None,
+                    help="with --ronavik: only this layer size")
+    ap.add_argument("--ronavik-design", choices=["both", "ronavik", "sabezen"], default="both",
+                    help="with --ronavik: only one of the two designs (for profiling)")
     ap.add_argument("--no-extra-points", action="store_true",
                     help="skip the other shapes and the longer context that the default run adds under `points`")
     return ap.parse_args(argv)
@@ -226,6 +243,17 @@ def sabezen_configs(size: dict, layers: int, vocab: int = 32000):
     return sab, llama
 
 
+def ronavik_config(size: dict, layers: int, vocab: int = 32000) -> dict:
+    d, H, G, hd = size["width"], size["heads"], size["kv_heads"], size["dim"]
+    pair = {"type": "parallel", "mixer": {
+        "left": {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "q_temp": {"coef": 0.1, "every": 1024}},
+        "right": {"width": d, "blocks": d // 256, "conv": 4}, "left_scale": 1.0, "right_scale": 1.0}}
+    ssm = {"type": "mamba2", "mixer": {"heads": 2 * d // 64, "vdim": 64, "state": 128, "groups": 8, "conv": 4, "norm_groups": 8}}
+    moe = {"kind": "moe", "expert": {"ff": size["expert_ff"]}, "router": {"experts": 16, "top": 2}}
+    return {"architecture": "Ronavik", "vocab": vocab, "width": d, "norm": {"eps": 1e-5}, "max_positions": 4096,
+            "layers": [dict((pair, ssm)[i % 2], mlp=moe) for i in range(layers)]}
+
+
 def design_point(cj: dict, batch: int, steps: int, warmup: int) -> dict:
     """Prefill of 2,048 tokens and decode at `batch` requests of 1,024-token prompts for any
     registered architecture: times, and the fractions of the HBM and matrix peaks by the bytes a
@@ -246,7 +274,7 @@ def design_point(cj: dict, batch: int, steps: int, warmup: int) -> dict:
     used, read = {}, {}
     for ls in spec.layers:
         f = ls.feed_forward
-        if f is not None and f.kind == "table_moe":
+        if f is not None and f.kind in ("table_moe", "routed_moe"):
             used[ls.name_of("feed_forward", "")] = f.get("top") / f.get("experts")
             read[ls.name_of("feed_forward", "")] = min(1.0, batch * f.get("top") / f.get("experts"))
 
@@ -258,16 +286,21 @@ def design_point(cj: dict, batch: int, steps: int, warmup: int) -> dict:
     chunked_flops = 0.0         # attention over chunks: the keys that a prompt of PREFILL tokens sees
     state_bytes = sum(4 * int(np.prod(shape)) for _, shape, dt in model.state_specs() if dt == torch.float32)
     scan_flops_a_token = 0      # the recurrences' multiply-adds on the vector units, counted apart
-    for ls in spec.layers:
-        m = ls.mixer
+    mixers = [m for ls in spec.layers for m in ((ls.mixer.get("left"), ls.mixer.get("right"))
+                                                if ls.mixer.kind == "side_by_side" else (ls.mixer,))]
+    for m in mixers:
         if m.kind == "mixed_attention":
             seen = sum(i % m.get("chunk") + 1 for i in range(PREFILL)) if m.get("chunk") else PREFILL * (PREFILL + 1) / 2
             chunked_flops += 2.0 * 2 * m.get("dim") * m.get("num_heads") * seen
         elif m.kind in ("gated_delta", "gla"):
             scan_flops_a_token += 2 * (4 if m.kind == "gated_delta" else 3) * m.get("num_heads") * m.get("dim") * m.get("vdim")
+        elif m.kind == "state_space":
+            scan_flops_a_token += 2 * 3 * m.get("num_heads") * m.get("state") * m.get("vdim")
+        elif m.kind == "rglru":      # the two gates' block products, in float32 on the vector units
+            scan_flops_a_token += 2 * 2 * m.get("width") * (m.get("width") // m.get("blocks"))
         if m.kind == "attention":
             attention_dims += 2 * m.get("head_dim") * m.get("num_heads")
-        elif m.kind == "kv_attention":
+        elif m.kind in ("kv_attention", "sigmoid_attention"):
             attention_dims += (m.get("key_dim") + m.get("value_dim")) * m.get("num_heads")
         elif m.kind == "latent_attention":
             attention_dims += (2 * m.get("kv_rank") + m.get("rotated_dim")) * m.get("num_heads")
@@ -343,6 +376,24 @@ def vofezen_compare(args) -> dict:
             "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16", "layers": layers, "points": points}
 
 
+def ronavik_compare(args) -> dict:
+    import hfee_amd  # noqa: F401
+    layers = args.layers or 6
+    points = {}
+    for name, size in RONAVIK_SIZES.items():
+        if args.ronavik_size not in (None, name):
+            continue
+        sab, _ = sabezen_configs(SABEZEN_SIZES[name], layers)
+        for design, cj in (("ronavik", ronavik_config(size, layers)), ("sabezen", sab)):
+            if args.ronavik_design not in ("both", design):
+                continue
+            print(f"[bench] {design} {name}, {layers} layers", file=sys.stderr, flush=True)
+            points[f"{design}_{name}"] = design_point(cj, args.batch, min(args.steps, 32), min(args.warmup, 4))
+    return {"metric": "Ronavik beside Sabezen at equal layer sizes: prefill of 2,048 tokens, decode at batch %d and "
+                      "1,024-token prompts (bf16, random weights)" % args.batch,
+            "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16", "layers": layers, "points": points}
+
+
 def sabezen_compare(args) -> dict:
     import hfee_amd  # noqa: F401
     layers = args.layers or 6
@@ -366,6 +417,9 @@ def main(argv=None) -> int:
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.ronavik:
+        print(json.dumps(ronavik_compare(args)), flush=True)
+        return 0
     if args.sabezen:
         print(json.dumps(sabezen_compare(args)), flush=True)
         return 0

@@ -59,7 +59,7 @@ def attention_mix_fits(heads: int, dim: int) -> bool:
 # other sizes compiles its own at first use)
 ATTENTION_KV_SIZES = ((32, 16), (64, 32), (96, 64), (48, 32), (16, 48), (112, 96), (64, 64), (160, 128), (128, 128), (576, 512))
 # the same for the kernels without a softmax
-ATTENTION_KV_SIGMOID_SIZES = ((32, 16), (16, 48), (32, 64), (128, 128))
+ATTENTION_KV_SIGMOID_SIZES = ((16, 32), (16, 48), (32, 64), (128, 128))
 
 
 class BuildError(RuntimeError):
