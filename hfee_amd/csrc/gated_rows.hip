@@ -7,7 +7,8 @@
 //                     y2 (a second mixer beside the first), the gate g with its bias c: each optional.
 //   scaled_add:       x += a y + b y2
 //
-// All sums in float32, one workgroup a row, a fixed order of additions.
+// All sums in float32, one workgroup a row, a fixed order of additions (which depends on the row's width and
+// alignment only, never on the other rows of the step).
 #include "common.h"
 
 using namespace hfee;
@@ -62,6 +63,99 @@ __global__ __launch_bounds__(256) void gated_norm_add_kernel(
     nr[j] = from_float<TN>(xr[j] * inv2 * w2[j]);
 }
 
+
+// The same for rows of up to 1024 * K values that are whole groups of four: a thread asks for all it needs of
+// the row at once (K groups of four of y, y2, the gate and x), keeps the gated values in registers between the
+// sum of squares and the addition, and the new row between the second sum and the following norm.  A row is
+// read once, and a step of a few rows is one wait for memory instead of one a loop turn.
+template <typename TG>
+__device__ __forceinline__ void load4(float (&v)[4], const TG* p);
+template <>
+__device__ __forceinline__ void load4<float>(float (&v)[4], const float* p) {
+  const float4 t = *reinterpret_cast<const float4*>(p);
+  v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+template <>
+__device__ __forceinline__ void load4<bf16_t>(float (&v)[4], const bf16_t* p) {
+  const uint2 t = *reinterpret_cast<const uint2*>(p);
+  v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+  v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+}
+template <typename TN>
+__device__ __forceinline__ void store4(TN* p, const float (&v)[4]);
+template <>
+__device__ __forceinline__ void store4<float>(float* p, const float (&v)[4]) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+template <>
+__device__ __forceinline__ void store4<bf16_t>(bf16_t* p, const float (&v)[4]) {
+  bf16_t h[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) h[i] = from_float<bf16_t>(v[i]);
+  *reinterpret_cast<uint2*>(p) = *reinterpret_cast<const uint2*>(h);
+}
+
+template <typename TG, typename TN, int K>
+__global__ __launch_bounds__(256) void gated_norm_add_held_kernel(
+    float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ y2, float a, float b,
+    const TG* __restrict__ gate, int64_t ldg, const float* __restrict__ gate_bias, const float* __restrict__ w, float eps,
+    TN* __restrict__ next, const float* __restrict__ w2, float eps2, int d) {
+  __shared__ float scratch[16];
+  const int64_t r = blockIdx.x;
+  float v[K][4], xs[K][4], ws[K][4];
+  {
+    float second[K][4], g[K][4], gb[K][4];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const int j = (k * 256 + threadIdx.x) * 4;
+      const bool in = j < d;
+      const int jj = in ? j : 0;
+      load4<float>(v[k], y + r * d + jj);
+      load4<float>(xs[k], x + r * d + jj);
+      load4<float>(ws[k], w + jj);
+      if (y2 != nullptr) load4<float>(second[k], y2 + r * d + jj);
+      if (gate != nullptr) load4<TG>(g[k], gate + r * ldg + jj);
+      if (gate_bias != nullptr) load4<float>(gb[k], gate_bias + jj);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float t = y2 != nullptr ? fmaf(a, v[k][i], b * second[k][i]) : a * v[k][i];
+        if (gate != nullptr) t *= 1.0f / (1.0f + expf(-(g[k][i] + (gate_bias != nullptr ? gb[k][i] : 0.f))));
+        v[k][i] = in ? t : 0.f;
+      }
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < K; ++k)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ss = fmaf(v[k][i], v[k][i], ss);
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+  float ss2 = 0.f;
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const int j = (k * 256 + threadIdx.x) * 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      xs[k][i] = j < d ? xs[k][i] + v[k][i] * inv * ws[k][i] : 0.f;
+      ss2 = fmaf(xs[k][i], xs[k][i], ss2);
+    }
+    if (j < d) store4<float>(x + r * d + j, xs[k]);
+  }
+  if (next == nullptr) return;
+  ss2 = block_sum(ss2, scratch);
+  const float inv2 = 1.0f / sqrtf(ss2 / (float)d + eps2);
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const int j = (k * 256 + threadIdx.x) * 4;
+    if (j >= d) continue;
+    load4<float>(ws[k], w2 + j);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) xs[k][i] = xs[k][i] * inv2 * ws[k][i];
+    store4<TN>(next + r * d + j, xs[k]);
+  }
+}
+
 }  // namespace
 
 HFEE_API int hfee_add_table_rows(float* x, int n, int d, const void* table, int dtype, const int* index, hipStream_t stream) {
@@ -85,10 +179,29 @@ HFEE_API int hfee_gated_norm_add(float* x, const float* y, const float* y2, floa
   HFEE_REQUIRE(next == nullptr || w2 != nullptr, "gated_norm_add: the following norm needs its weight");
   HFEE_REQUIRE(gate == nullptr || ldg >= d, "gated_norm_add: the gate's rows are too short");
   if (n == 0) return 0;
-#define LAUNCH(TG, TN)                                                                                               \
-  gated_norm_add_kernel<TG, TN><<<n, 256, 0, stream>>>(x, y, y2, a, b, (const TG*)gate, ldg, gate_bias, w, eps,      \
-                                                       (TN*)next, w2, eps2, d)
+  const auto aligned = [](const void* p, int to) { return (reinterpret_cast<uintptr_t>(p) & (uintptr_t)(to - 1)) == 0; };
+  const bool held = d % 4 == 0 && d <= 8192 && aligned(x, 16) && aligned(y, 16) && aligned(y2, 16) && aligned(w, 16) &&
+                    aligned(gate_bias, 16) && aligned(w2, 16) && aligned(next, 16) &&
+                    (gate == nullptr || (ldg % 4 == 0 && aligned(gate, 16)));
   const int code = (gate_dtype & 1) | ((next_dtype & 1) << 1);
+#define LAUNCH(TG, TN)                                                                                               \
+  do {                                                                                                               \
+    if (!held)                                                                                                       \
+      gated_norm_add_kernel<TG, TN><<<n, 256, 0, stream>>>(x, y, y2, a, b, (const TG*)gate, ldg, gate_bias, w, eps,  \
+                                                           (TN*)next, w2, eps2, d);                                  \
+    else if (d <= 1024)                                                                                              \
+      gated_norm_add_held_kernel<TG, TN, 1><<<n, 256, 0, stream>>>(x, y, y2, a, b, (const TG*)gate, ldg, gate_bias,  \
+                                                                   w, eps, (TN*)next, w2, eps2, d);                  \
+    else if (d <= 2048)                                                                                              \
+      gated_norm_add_held_kernel<TG, TN, 2><<<n, 256, 0, stream>>>(x, y, y2, a, b, (const TG*)gate, ldg, gate_bias,  \
+                                                                   w, eps, (TN*)next, w2, eps2, d);                  \
+    else if (d <= 4096)                                                                                              \
+      gated_norm_add_held_kernel<TG, TN, 4><<<n, 256, 0, stream>>>(x, y, y2, a, b, (const TG*)gate, ldg, gate_bias,  \
+                                                                   w, eps, (TN*)next, w2, eps2, d);                  \
+    else                                                                                                             \
+      gated_norm_add_held_kernel<TG, TN, 8><<<n, 256, 0, stream>>>(x, y, y2, a, b, (const TG*)gate, ldg, gate_bias,  \
+                                                                   w, eps, (TN*)next, w2, eps2, d);                  \
+  } while (0)
   if (code == 0) LAUNCH(float, float);
   else if (code == 1) LAUNCH(bf16_t, float);
   else if (code == 2) LAUNCH(float, bf16_t);

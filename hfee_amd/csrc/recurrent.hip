@@ -372,6 +372,13 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(T* __restrict__ out
 // to give the decay's logarithm (not positive).
 constexpr int kRgTokens = 8;
 
+__device__ __forceinline__ void rglru_token(float& decay, float& inject, float r, float g, float x, float bias_r,
+                                            float bias_i, float rt) {
+  const float log_a = rt / (1.0f + expf(-(r + bias_r)));
+  decay = expf(log_a);
+  inject = sqrtf(-expm1f(2.0f * log_a)) * x / (1.0f + expf(-(g + bias_i)));
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void rglru_scan_kernel(
     T* __restrict__ out, int64_t ldo, float* __restrict__ state, const float* __restrict__ gates, int64_t ldg,
@@ -398,10 +405,8 @@ __global__ __launch_bounds__(256) void rglru_scan_kernel(
     }
 #pragma unroll
     for (int j = 0; j < kRgTokens; ++j) {
-      const float log_a = rt / (1.0f + expf(-(r[j] + bias_r)));
-      r[j] = expf(log_a);
       // 1 - a^2 = -(exp(2 log a) - 1): no cancellation where the decay is close to one
-      g[j] = sqrtf(-expm1f(2.0f * log_a)) * x[j] / (1.0f + expf(-(g[j] + bias_i)));
+      rglru_token(r[j], g[j], r[j], g[j], x[j], bias_r, bias_i, rt);
       const float v = z[j] + yb;
       z[j] = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
     }
@@ -414,6 +419,109 @@ __global__ __launch_bounds__(256) void rglru_scan_kernel(
     }
   }
   *sp = S;
+}
+
+// The same unit for long portions, cut into chunks of kRgChunk tokens so that a portion of thousands of tokens
+// is walked by as many threads as it has (channel, chunk) pairs instead of one a channel.  A chunk's tokens
+// act on what comes into it as S -> P S + Q with P the product of its decays and Q its walk from zero:
+//   chunk_ends   every chunk but a portion's last: P and Q, and the slot's state set aside (`starts`);
+//   chunk_walk   a chunk's incoming S from `starts` through the chunks before it, one multiply-add a chunk in
+//                their order (every thread of a channel does the same sums, so they agree on each chunk's
+//                S to the bit); then the walk over its own tokens as in rglru_scan; the last chunk leaves
+//                the state.
+// ends: float32 [segments][chunks_most][2][W]; starts: float32 [segments][W].  Chunks count from the
+// portion's first token, so how a prompt was cut moves the roundings of P S + Q and nothing else.
+constexpr int kRgChunk = 32;
+
+__global__ __launch_bounds__(256) void rglru_chunk_ends_kernel(
+    float* __restrict__ ends, float* __restrict__ starts, int chunks_most, const float* __restrict__ state,
+    const float* __restrict__ gates, int64_t ldg, const float* __restrict__ gate_bias, const float* __restrict__ u,
+    int64_t ldu, const float* __restrict__ rate, const int* __restrict__ segment_rows,
+    const int* __restrict__ segment_lengths, const int* __restrict__ segment_slots, int W, int block) {
+  const int seg = blockIdx.z, chunk = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int len = segment_lengths[seg], first = chunk * kRgChunk;
+  if (c >= W || first >= len) return;
+  if (chunk == 0) starts[(int64_t)seg * W + c] = state[(int64_t)segment_slots[seg] * W + c];
+  if (first + kRgChunk >= len) return;          // (nothing comes behind a portion's last chunk)
+  const int b = c / block, at_r = b * 2 * block + (c - b * block), at_i = at_r + block;
+  const float bias_r = gate_bias[at_r], bias_i = gate_bias[at_i], rt = rate[c];
+  const int64_t row0 = segment_rows[seg] + first;
+  float P = 1.f, Q = 0.f;
+  for (int t = 0; t < kRgChunk; t += kRgTokens) {
+    float r[kRgTokens], g[kRgTokens], x[kRgTokens];
+#pragma unroll
+    for (int j = 0; j < kRgTokens; ++j) {
+      const int64_t row = row0 + t + j;
+      r[j] = gates[row * ldg + at_r];
+      g[j] = gates[row * ldg + at_i];
+      x[j] = u[row * ldu + c];
+    }
+#pragma unroll
+    for (int j = 0; j < kRgTokens; ++j) rglru_token(r[j], g[j], r[j], g[j], x[j], bias_r, bias_i, rt);
+#pragma unroll
+    for (int j = 0; j < kRgTokens; ++j) {
+      P *= r[j];
+      Q = fmaf(r[j], Q, g[j]);
+    }
+  }
+  float* e = ends + ((int64_t)seg * chunks_most + chunk) * 2 * W + c;
+  e[0] = P;
+  e[W] = Q;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rglru_chunk_walk_kernel(
+    T* __restrict__ out, int64_t ldo, float* __restrict__ state, const float* __restrict__ ends,
+    const float* __restrict__ starts, int chunks_most, const float* __restrict__ gates, int64_t ldg,
+    const float* __restrict__ gate_bias, const float* __restrict__ u, int64_t ldu, const float* __restrict__ rate,
+    const T* __restrict__ y, int64_t ldy, const float* __restrict__ y_bias, const int* __restrict__ segment_rows,
+    const int* __restrict__ segment_lengths, const int* __restrict__ segment_slots, int W, int block) {
+  const int seg = blockIdx.z, chunk = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int len = segment_lengths[seg], first = chunk * kRgChunk;
+  if (c >= W || first >= len) return;
+  const int b = c / block, at_r = b * 2 * block + (c - b * block), at_i = at_r + block;
+  const float bias_r = gate_bias[at_r], bias_i = gate_bias[at_i], rt = rate[c], yb = y_bias != nullptr ? y_bias[c] : 0.f;
+  float S = starts[(int64_t)seg * W + c];
+  const float* e = ends + (int64_t)seg * chunks_most * 2 * W + c;
+  for (int k = 0; k < chunk; k += 8) {
+    float P[8], Q[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int kk = k + j < chunk ? k + j : k;
+      P[j] = e[(int64_t)kk * 2 * W];
+      Q[j] = e[(int64_t)kk * 2 * W + W];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (k + j < chunk) S = fmaf(P[j], S, Q[j]);
+  }
+  const int64_t row0 = segment_rows[seg] + first;
+  const int count = len - first < kRgChunk ? len - first : kRgChunk;
+  for (int t = 0; t < count; t += kRgTokens) {
+    float r[kRgTokens], g[kRgTokens], x[kRgTokens], z[kRgTokens];
+#pragma unroll
+    for (int j = 0; j < kRgTokens; ++j) {
+      const int64_t row = row0 + t + (t + j < count ? j : 0);
+      r[j] = gates[row * ldg + at_r];
+      g[j] = gates[row * ldg + at_i];
+      x[j] = u[row * ldu + c];
+      z[j] = to_float<T>(y[row * ldy + c]);
+    }
+#pragma unroll
+    for (int j = 0; j < kRgTokens; ++j) {
+      rglru_token(r[j], g[j], r[j], g[j], x[j], bias_r, bias_i, rt);
+      const float v = z[j] + yb;
+      z[j] = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+    }
+#pragma unroll
+    for (int j = 0; j < kRgTokens; ++j) {
+      if (t + j < count) {
+        S = fmaf(r[j], S, g[j]);
+        out[(row0 + t + j) * ldo + c] = from_float<T>(S * z[j]);
+      }
+    }
+  }
+  if (first + kRgChunk >= len) state[(int64_t)segment_slots[seg] * W + c] = S;
 }
 
 // One workgroup a (token, part).  o: float32 [n, inner], what the recurrence read; x: float32 [n, inner],
@@ -563,24 +671,45 @@ HFEE_API int hfee_head_norm_gate(void* out, int64_t ldo, const float* o, int64_t
   return 0;
 }
 
+// longest: the step's longest portion (host).  Portions of more than 2 * kRgChunk tokens go through the kernels
+// in chunks, which need (segments * ceil(longest / kRgChunk) * 2 + segments) * width floats of scratch.
 HFEE_API int hfee_rglru_scan(void* out, int64_t ldo, int dtype, float* state, const float* gates, int64_t ldg,
                              const float* gate_bias, const float* u, int64_t ldu, const float* rate, const void* y,
                              int64_t ldy, const float* y_bias, const int* segment_rows, const int* segment_lengths,
-                             const int* segment_slots, int segments, int width, int block, hipStream_t stream) {
+                             const int* segment_slots, int segments, int width, int block, int longest, float* scratch,
+                             int64_t scratch_floats, hipStream_t stream) {
   HFEE_REQUIRE(segments >= 0 && segments <= 65535 && width > 0 && block > 0 && width % block == 0,
                "rglru_scan: %d channels are not whole blocks of %d", width, block);
   HFEE_REQUIRE(ldo >= width && ldu >= width && ldy >= width && ldg >= 2 * (int64_t)width, "rglru_scan: rows too short");
   HFEE_REQUIRE(gate_bias != nullptr && rate != nullptr, "rglru_scan: the gates' biases and the decay's rates");
+  HFEE_REQUIRE(dtype == 0 || dtype == 1, "rglru_scan: unknown dtype %d", dtype);
   if (segments == 0) return 0;
+  if (longest > 2 * kRgChunk && scratch != nullptr) {
+    const int chunks_most = (longest + kRgChunk - 1) / kRgChunk;
+    HFEE_REQUIRE(chunks_most <= 65535 && ((int64_t)segments * chunks_most * 2 + segments) * width <= scratch_floats,
+                 "rglru_scan: %lld floats of scratch do not hold %d portions of up to %d chunks", (long long)scratch_floats,
+                 segments, chunks_most);
+    float* starts = scratch + (int64_t)segments * chunks_most * 2 * width;
+    dim3 grid((width + 255) / 256, chunks_most, segments);
+    rglru_chunk_ends_kernel<<<grid, 256, 0, stream>>>(scratch, starts, chunks_most, state, gates, ldg, gate_bias, u, ldu,
+                                                      rate, segment_rows, segment_lengths, segment_slots, width, block);
+    HFEE_CHECK_LAUNCH("rglru_scan (chunk ends)");
+    if (dtype == 0)
+      rglru_chunk_walk_kernel<float><<<grid, 256, 0, stream>>>((float*)out, ldo, state, scratch, starts, chunks_most, gates,
+          ldg, gate_bias, u, ldu, rate, (const float*)y, ldy, y_bias, segment_rows, segment_lengths, segment_slots, width, block);
+    else
+      rglru_chunk_walk_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out, ldo, state, scratch, starts, chunks_most, gates,
+          ldg, gate_bias, u, ldu, rate, (const bf16_t*)y, ldy, y_bias, segment_rows, segment_lengths, segment_slots, width, block);
+    HFEE_CHECK_LAUNCH("rglru_scan (chunk walk)");
+    return 0;
+  }
   dim3 grid((width + 255) / 256, segments);
   if (dtype == 0)
     rglru_scan_kernel<float><<<grid, 256, 0, stream>>>((float*)out, ldo, state, gates, ldg, gate_bias, u, ldu, rate,
         (const float*)y, ldy, y_bias, segment_rows, segment_lengths, segment_slots, width, block);
-  else if (dtype == 1)
+  else
     rglru_scan_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out, ldo, state, gates, ldg, gate_bias, u, ldu, rate,
         (const bf16_t*)y, ldy, y_bias, segment_rows, segment_lengths, segment_slots, width, block);
-  else
-    return fail("rglru_scan: unknown dtype %d", dtype);
   HFEE_CHECK_LAUNCH("rglru_scan");
   return 0;
 }

@@ -61,7 +61,7 @@ _CORE_SIGNATURES = {
     "hfee_unit_heads": [P, L, I, I, F, F, I, P],
     "hfee_scan_gate": [P, L, P, L, I, P, P, I, I, F, I, I, I, P],
     "hfee_linear_scan": [P, L, P, P, L, P, L, P, L, P, L, P, L, P, P, P, I, I, I, I, I, I, I, P],
-    "hfee_rglru_scan": [P, L, I, P, P, L, P, P, L, P, P, L, P, P, P, P, I, I, I, P],
+    "hfee_rglru_scan": [P, L, I, P, P, L, P, P, L, P, P, L, P, P, P, P, I, I, I, I, P, L, P],
     "hfee_gate_group_norm": [P, L, I, P, L, P, L, P, I, P, L, P, I, I, F, I, P],
     "hfee_router_topk": [P, L, I, I, I, P, P, P],
     "hfee_add_table_rows": [P, I, I, P, I, P, P],

@@ -1346,12 +1346,25 @@ def linear_scan(out, state, q, k, v, decay, beta, segment_rows, segment_lengths,
                     _ptr(segment_slots), segments, heads, qk_heads, dim, vdim, rules[rule], 1 if decay_per_head else 0, _stream())
 
 
-def rglru_scan(out, state, gates, gate_bias, u, rate, y, y_bias, segment_rows, segment_lengths, segment_slots, block: int):
+RGLRU_CHUNK = 32        # tokens a chunk of the recurrent unit's kernels for long portions
+
+
+def rglru_scan_scratch(longest: int, segments: int, width: int) -> int:
+    """float32 words that `rglru_scan` needs for a step whose longest portion has `longest` tokens."""
+    if longest <= 2 * RGLRU_CHUNK:
+        return 0
+    return (segments * (-(-longest // RGLRU_CHUNK)) * 2 + segments) * width
+
+
+def rglru_scan(out, state, gates, gate_bias, u, rate, y, y_bias, segment_rows, segment_lengths, segment_slots, block: int,
+               longest: int = 0, scratch=None):
     """The real-gated linear recurrent unit, a number a channel: with r, i the gates of a token (gates:
     float32 [n, blocks, 2 * block] before bias and sigmoid, a block's r, then its i; gate_bias float32 of
     that width), a = exp(rate * sigmoid(r)) (rate float32 [W], not positive),
     S <- a S + sqrt(1 - a^2) sigmoid(i) u, out = S * gelu_tanh(y + y_bias) in y's dtype.  state: float32
-    [slots, W], walked from and left in each segment's slot; u float32 [n, W]; y [n, W]."""
+    [slots, W], walked from and left in each segment's slot; u float32 [n, W]; y [n, W].  longest: the
+    longest portion of the step, if known; with `scratch` (float32, `rglru_scan_scratch` words) long
+    portions are walked in chunks by many threads a channel."""
     _gpu(out, state, gates, gate_bias, u, rate, y, y_bias, segment_rows, segment_lengths, segment_slots)
     n, W, ldu = _f32rows(u, "rglru_scan u")
     ng, wg, ldg = _f32rows(gates, "rglru_scan gates")
@@ -1366,9 +1379,15 @@ def rglru_scan(out, state, gates, gate_bias, u, rate, y, y_bias, segment_rows, s
     _i32(segment_rows, "rglru_scan segment_rows")
     _i32(segment_lengths, "rglru_scan segment_lengths", segments)
     _i32(segment_slots, "rglru_scan segment_slots", segments)
+    words = 0
+    if scratch is not None:
+        _gpu(scratch)
+        _check(scratch.dtype == torch.float32 and scratch.is_contiguous(), "rglru_scan: scratch float32")
+        _check(0 < longest <= n, "rglru_scan: scratch comes with the longest portion's length")
+        words = scratch.numel()
     lib.core().call("hfee_rglru_scan", _ptr(out), ldo, _dt(out), _ptr(state), _ptr(gates), ldg, _ptr(gate_bias), _ptr(u), ldu,
                     _ptr(rate), _ptr(y), ldy, _ptr(y_bias), _ptr(segment_rows), _ptr(segment_lengths), _ptr(segment_slots),
-                    segments, W, int(block), _stream())
+                    segments, W, int(block), int(longest), _ptr(scratch), words, _stream())
 
 
 def gate_group_norm(out, o, x, skip, z, weight, heads: int, parts: int, eps: float):

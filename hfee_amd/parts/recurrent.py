@@ -360,7 +360,11 @@ class RealGatedRecurrentUnit(_StateMixer):
         gates = ctx.rows("rglru.gates", 2 * W, torch.float32)
         ops.head_linear(gates, u, self.w_gates, self.blocks, self.block, 2 * self.block)
         read = ctx.rows("rglru.read", W)
-        ops.rglru_scan(read, self.state, gates, self.gate_bias, u, self.rate, y, self.y_bias, rows, lengths, slots, self.block)
+        longest = max(s.length for s in ctx.segments)
+        words = ops.rglru_scan_scratch(longest, len(ctx.segments), W)
+        scratch = ctx.workspace.flat("rglru.chunks", words, torch.float32) if words else None
+        ops.rglru_scan(read, self.state, gates, self.gate_bias, u, self.rate, y, self.y_bias, rows, lengths, slots, self.block,
+                       longest=longest, scratch=scratch)
         product(ctx, out, read, self.w_o, self.w_o_tiles)
 
     def forward_add(self, ctx, x, h, cache_layer: int, writes_cache: bool):

@@ -110,12 +110,21 @@ def state_space(h, w, pre, m, eps):
     return (yg.reshape(T, inner) * w[pre + "norm"]) @ w[pre + "o"].T
 
 
-def routed_experts(h, w, pre, mlp):
+def routed_experts(h, w, pre, mlp, margins=None):
     """Scores sigmoid(W_router h); the `top` largest choose the experts; a chosen expert's score
-    multiplies its input; down(relu(up(.))^2); the outputs are summed."""
+    multiplies its input; down(relu(up(.))^2); the outputs are summed.  margins: a list that receives, a
+    token, how far the last chosen expert's logit is above the best one not chosen, in units of the
+    logits' spread over the experts (infinite where every expert is chosen)."""
     E, top = mlp["router"]["experts"], mlp["router"]["top"]
-    s = torch.sigmoid(h @ w[pre + "router"].T)
+    z = h @ w[pre + "router"].T
+    s = torch.sigmoid(z)
     vals, idx = torch.topk(s, top, dim=-1)
+    if margins is not None:
+        if top < E:
+            best = torch.topk(z, top + 1, dim=-1).values
+            margins.append((best[:, top - 1] - best[:, top]) / z.std(dim=-1).clamp_min(1e-30))
+        else:
+            margins.append(torch.full((h.shape[0],), float("inf"), dtype=h.dtype))
     out = torch.zeros(h.shape[0], w[pre + "e0.down"].shape[0], dtype=h.dtype)
     for t in range(h.shape[0]):
         for j in range(top):
@@ -125,9 +134,9 @@ def routed_experts(h, w, pre, mlp):
     return out
 
 
-def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, layers_out=None):
+def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, layers_out=None, margins_out=None):
     """Logits [T, vocab] of one sequence from position 0.  layers_out: a list that receives the
-    residual stream after every layer."""
+    residual stream after every layer; margins_out: one that receives every router's margins [T]."""
     w = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in w.items()}
     eps = cfg["norm"]["eps"]
     tok = torch.as_tensor(tokens, dtype=torch.long)
@@ -145,7 +154,7 @@ def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, layers_out=None):
         x = x + rms_norm(y, w[pre + "norm1b"], eps)
         if layer.get("mlp") is not None:
             h = rms_norm(x, w[pre + "norm2"], eps)
-            y = routed_experts(h, w, pre + "mlp.", layer["mlp"])
+            y = routed_experts(h, w, pre + "mlp.", layer["mlp"], margins_out)
             y = y * torch.sigmoid(h @ w[pre + "rg2"].T + w[pre + "rg2.b"])
             x = x + rms_norm(y, w[pre + "norm2b"], eps)
         if layers_out is not None:

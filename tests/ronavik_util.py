@@ -62,7 +62,17 @@ R_D = config(500, 128, 1e-6, 1024, [
     moe(ssm(4, 32, 32, 2, 3, 2), 96, 8, 1),
     moe(pair(8, 2, 32, 64, 0.15, 128, 4, 3, q_temp=(0.3, 64), left_scale=1.1, right_scale=0.8), 64, 8, 2),
 ])
-CONFIGS = {"A": R_A, "B": R_B, "C": R_C, "D": R_D}
+
+
+def every_expert(cj):
+    """The same configuration with routers that choose every expert for every token."""
+    layers = [layer if layer["mlp"] is None else
+              dict(layer, mlp=dict(layer["mlp"], router=dict(layer["mlp"]["router"], top=layer["mlp"]["router"]["experts"])))
+              for layer in cj["layers"]]
+    return dict(cj, layers=layers)
+
+
+CONFIGS = {"A": R_A, "B": R_B, "C": R_C, "D": R_D, "A every expert": every_expert(R_A), "D every expert": every_expert(R_D)}
 
 # one mechanism each (a pair with one of its scales zero is the other mixer alone)
 SINGLE = {

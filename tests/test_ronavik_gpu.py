@@ -146,7 +146,7 @@ def test_the_temperature_steps_where_it_should():
     """q at positions around multiples of `every`: the factor is 1 + coef * ln(floor((p + 1) / every) + 1)."""
     from hfee_amd.kernels import ops
     every, coef, dk = 7, 0.9, 8
-    positions = [0, 5, 6, 7, 12, 13, 14, 48, 49]
+    positions = [0, 5, 6, 7, 12, 13, 14, 47, 48]
     q = torch.ones(len(positions), dk).cuda()
     ops.qk_norm_write(q, None, None, i32(positions), None, None, None, torch.ones(dk).cuda(), None, 0.0, 1, 1, dk, dk, 16,
                       temperature=(coef, every))
@@ -159,11 +159,12 @@ def test_the_temperature_steps_where_it_should():
 @pytest.mark.parametrize("W,blocks", [(48, 3), (40, 1), (300, 5)])
 def test_recurrent_unit_in_portions(dtype, W, blocks):
     """The unit by its definition in float64 against the kernels fed the same two sequences in portions of
-    unequal size (down to single tokens) in other slots; a slot of NaNs beside them stays untouched."""
+    unequal size (down to single tokens, and long ones that are walked in chunks, the last chunk not full,
+    beside a short one) in other slots; a slot of NaNs beside them stays untouched."""
     from hfee_amd.kernels import ops
     dt = DT[dtype]
     g = torch.Generator().manual_seed(W)
-    T, bs = [45, 23], W // blocks
+    T, bs = [301, 23], W // blocks
     ra, ri = torch.randn(blocks, bs, bs, generator=g) * 0.5, torch.randn(blocks, bs, bs, generator=g) * 0.5
     rab, rib = torch.randn(blocks, bs, generator=g), torch.randn(blocks, bs, generator=g)
     lam, yb = torch.randn(W, generator=g) - 2.0, torch.randn(W, generator=g) * 0.3
@@ -188,7 +189,7 @@ def test_recurrent_unit_in_portions(dtype, W, blocks):
     state[1].fill_(float("nan"))
     slots, fed = [3, 0], [0, 0]
     got = [torch.zeros(t, W) for t in T]
-    for sizes in ([7, 2], [1, 1], [20, 0], [2, 13], [15, 7]):
+    for sizes in ([7, 2], [1, 1], [150, 0], [2, 13], [141, 7]):
         segs = [(s, n) for s, n in enumerate(sizes) if n]
         u = torch.cat([us[s][fed[s]:fed[s] + n] for s, n in segs]).cuda()
         y = torch.cat([ys[s][fed[s]:fed[s] + n] for s, n in segs]).to(dt).cuda()
@@ -196,8 +197,11 @@ def test_recurrent_unit_in_portions(dtype, W, blocks):
         gates = torch.zeros(u.shape[0], 2 * W, device="cuda")
         ops.head_linear(gates, u, w_gates, blocks, bs, 2 * bs)
         out = torch.zeros(u.shape[0], W, dtype=dt, device="cuda")
+        words = ops.rglru_scan_scratch(max(sizes), len(segs), W)
+        assert (words > 0) == (max(sizes) > 100)
         ops.rglru_scan(out, state, gates, gate_bias, u, rate, y, yb.cuda(), i32(rows), i32([n for _, n in segs]),
-                       i32([slots[s] for s, _ in segs]), bs)
+                       i32([slots[s] for s, _ in segs]), bs, longest=max(sizes),
+                       scratch=torch.full((words,), float("nan"), device="cuda") if words else None)
         for (s, n), r in zip(segs, rows):
             got[s][fed[s]:fed[s] + n] = out[r:r + n].float().cpu()
             fed[s] += n
@@ -296,23 +300,28 @@ def test_gate_then_norm_in_parts_and_the_gated_residual(dtype):
     yg = y.view(n, parts, -1)
     want = (yg / torch.sqrt((yg * yg).mean(-1, keepdim=True) + eps)).reshape(n, inner) * w.double()
     assert ru.rel(out.double().cpu(), want) < (2e-6 if dtype == "float32" else 6e-3)
-    # x += norm((a y + b y2) * sigmoid(gate + bias)) * w, and the norm that follows
+    # x += norm((a y + b y2) * sigmoid(gate + bias)) * w, and the norm that follows: rows that are no whole
+    # groups of four or start anywhere (a loop over the row), and rows that a thread holds in registers
+    # (one, two and eight groups a thread, the last ones past the row's end)
+    for d, shift in ((90, 3), (64, 8), (1032, 8), (5000, 16)):
+        xs, y1, y2 = (torch.randn(n, d, generator=g) for _ in range(3))
+        wide = torch.randn(n, d + 2 * shift, generator=g).to(dt)
+        gate, gate_gpu = wide[:, shift:shift + d], wide.cuda()[:, shift:shift + d]        # (rows inside wider rows)
+        gb, w1, w2 = torch.randn(d, generator=g), torch.rand(d, generator=g) + 0.5, torch.rand(d, generator=g) + 0.5
+        for second in (True, False):
+            for gated in (True, False):
+                xg, nxt = xs.clone().cuda(), torch.zeros(n, d, dtype=dt, device="cuda")
+                ops.gated_norm_add(xg, y1.cuda(), w1.cuda(), eps, y2=y2.cuda() if second else None, scales=(0.7, -1.3),
+                                   gate=gate_gpu if gated else None, gate_bias=gb.cuda() if gated else None, next_out=nxt,
+                                   next_weight=w2.cuda(), next_eps=2 * eps)
+                v = 0.7 * y1.double() + (-1.3 * y2.double() if second else 0)
+                if gated:
+                    v = v * torch.sigmoid(gate.double() + gb.double())
+                want_x = xs.double() + pr.rms_norm(v, w1.double(), eps)
+                assert ru.rel(xg.double().cpu(), want_x) < 2e-6
+                assert ru.rel(nxt.double().cpu(), pr.rms_norm(want_x, w2.double(), 2 * eps)) < (2e-6 if dtype == "float32" else 6e-3)
     d = 90
     xs, y1, y2 = (torch.randn(n, d, generator=g) for _ in range(3))
-    gate = torch.randn(n, d + 6, generator=g).to(dt)[:, 3:3 + d]
-    gb, w1, w2 = torch.randn(d, generator=g), torch.rand(d, generator=g) + 0.5, torch.rand(d, generator=g) + 0.5
-    for second in (True, False):
-        for gated in (True, False):
-            xg, nxt = xs.clone().cuda(), torch.zeros(n, d, dtype=dt, device="cuda")
-            ops.gated_norm_add(xg, y1.cuda(), w1.cuda(), eps, y2=y2.cuda() if second else None, scales=(0.7, -1.3),
-                               gate=gate.cuda() if gated else None, gate_bias=gb.cuda() if gated else None, next_out=nxt,
-                               next_weight=w2.cuda(), next_eps=2 * eps)
-            v = 0.7 * y1.double() + (-1.3 * y2.double() if second else 0)
-            if gated:
-                v = v * torch.sigmoid(gate.double() + gb.double())
-            want_x = xs.double() + pr.rms_norm(v, w1.double(), eps)
-            assert ru.rel(xg.double().cpu(), want_x) < 2e-6
-            assert ru.rel(nxt.double().cpu(), pr.rms_norm(want_x, w2.double(), 2 * eps)) < (2e-6 if dtype == "float32" else 6e-3)
     xa = xs.clone().cuda()
     ops.scaled_add(xa, y1.cuda(), 0.7, y2.cuda(), -1.3)
     assert ru.rel(xa.cpu(), xs + 0.7 * y1 - 1.3 * y2) < 1e-6
@@ -376,9 +385,29 @@ def folders(tmp_path_factory):
             for name, cj in list(ru.CONFIGS.items()) + list(ru.SINGLE.items()) for dtype in ("float32", "bfloat16")}
 
 
-def plain_logits(folder, tokens):
+def plain_logits(folder, tokens, margins=None):
+    """The plain implementation's logits; margins: a list that receives, a position, the smallest margin by
+    which any of its routers chose."""
     cj, w = ru.load_plain(folder)
-    return pr.forward(cj, w, tokens, dtype=torch.float64).numpy()
+    each = []
+    logits = pr.forward(cj, w, tokens, dtype=torch.float64, margins_out=each).numpy()
+    if margins is not None:
+        margins.extend(torch.stack(each).min(0).values.tolist() if each else [float("inf")] * len(tokens))
+    return logits
+
+
+# In bfloat16 a router reads rounded numbers: a token whose last chosen expert and the best one not chosen
+# score almost alike may go to the other one.  Its sub-layer's result is normed, so that is a change as large
+# as the stream itself, and the states and the cache carry it to every token behind it.  So in bfloat16 a
+# request is compared up to the first position at which a router of the plain implementation chose by less
+# than NEAR_TIE of its logits' spread (a few positions in a hundred), and the configurations in which every
+# token uses every expert ("... every expert": nothing is chosen) are compared at every position.
+NEAR_TIE = 0.05
+
+
+class Rows(dict):
+    """(request, position) -> logits of the plain implementation; `.margins`: -> the routers' smallest margin."""
+    margins: dict
 
 
 @pytest.fixture(scope="module")
@@ -386,29 +415,42 @@ def plain_rows(folders):
     cache = {}
 
     def get(name, dtype, lengths=None):
-        key = (name, dtype, tuple(lengths or LENGTHS[name]))
+        key = (name, dtype, tuple(lengths or LENGTHS[name[0]]))
         if key not in cache:
             cj = (ru.CONFIGS.get(name) or ru.SINGLE[name])
             reqs = tu.make_requests(cj["vocab"], list(key[2]), seed=ord(name[0]))
-            rows = {}
+            rows = Rows()
+            rows.margins = {}
             for rid, toks in reqs.items():
-                logits = plain_logits(folders[(name, dtype)], toks)
+                margins = []
+                logits = plain_logits(folders[(name, dtype)], toks, margins)
                 rows.update({(rid, i): logits[i] for i in range(len(toks))})
+                rows.margins.update({(rid, i): margins[i] for i in range(len(toks))})
             cache[key] = (reqs, rows)
         return cache[key]
     return get
 
 
-def compare(got, want, dtype, what):
-    """In 32-bit every position is within the tolerance.  In bfloat16 a token whose two best experts score
-    almost alike may go to the other one (the router reads rounded numbers): at most one position in fifty
-    may be beyond the tolerance, and the median is well within it."""
+def compare(got, want, dtype, what, margins=None):
+    """32-bit: every position within the tolerance.  bfloat16: every position before its request's first near
+    tie (see NEAR_TIE) within twice the tolerance and all but one in two hundred of them within it (rounding
+    has outliers where a row of logits is small); over all positions, also those behind a near tie, the
+    median is well within it."""
     assert set(got) == set(want), f"{what}: positions differ"
     tol = TOL[dtype]
+    margins = margins if margins is not None else getattr(want, "margins", {})
     errors = {key: ru.rel(got[key], want[key]) for key in want}
-    over = sorted((e, key) for key, e in errors.items() if not e < tol)
-    allowed = 0 if dtype == "float32" else max(1, len(want) // 50)
-    assert len(over) <= allowed, f"{what}: {len(over)} of {len(want)} positions beyond {tol}, the worst {over[-1]}"
+    keys = sorted(want)
+    if dtype != "float32":
+        first_tie = {}
+        for rid, at in keys:
+            if margins.get((rid, at), float("inf")) < NEAR_TIE:
+                first_tie[rid] = min(at, first_tie.get(rid, at))
+        keys = [(rid, at) for rid, at in keys if at < first_tie.get(rid, at + 1)]
+    over = sorted((errors[key], key) for key in keys if not errors[key] < tol)
+    allowed = 0 if dtype == "float32" else len(keys) // 200
+    assert len(over) <= allowed and not any(e >= 2 * tol for e, _ in over), \
+        f"{what}: {len(over)} of {len(keys)} positions beyond {tol}, the worst {over[-1]}, the first {min(k for _, k in over)}"
     assert np.median(list(errors.values())) < tol / 2, f"{what}: median relative error {np.median(list(errors.values())):.3e}"
 
 
@@ -423,15 +465,15 @@ def test_each_mechanism_as_a_model_of_one_layer(folders, plain_rows, name, dtype
         compare(tu.run(rep, steps), want, dtype, f"{name} {dtype} {what}")
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name,dtype", [(n, d) for n in ("A", "B", "C", "D") for d in ("float32", "bfloat16")]
+                         + [("A every expert", "bfloat16"), ("D every expert", "bfloat16")])
 def test_every_way_of_cutting_gives_the_plain_logits(folders, plain_rows, name, dtype):
     from hfee_amd.trace_replay import Replayer
     reqs, want = plain_rows(name, dtype)
     longest = max(len(t) for t in reqs.values())
     one = (longest + 63) // 64 * 64
     for what, steps, room in (("whole", tu.whole(reqs), one), ("bulk then single tokens", tu.bulk_then_tail(reqs, 40), one),
-                              ("portions", tu.portions(reqs), one), ("mixed", *tu.mixed(reqs, seed=len(name)))):
+                              ("portions", tu.portions(reqs), one), ("mixed", *tu.mixed(reqs, seed=len(name[0])))):
         rep = Replayer(folders[(name, dtype)], dtype, room, max_requests=4)
         got = tu.run(rep, steps)
         compare(got, want, dtype, f"{name} {dtype} {what}")
@@ -470,13 +512,16 @@ def test_long_decoding(folders, dtype):
     from hfee_amd.trace_replay import Replayer
     rng = np.random.default_rng(9)
     toks = rng.integers(0, 500, size=330).tolist()
-    rep = Replayer(folders[("D", dtype)], dtype, 384, max_requests=4)
+    name = "D" if dtype == "float32" else "D every expert"      # (in bfloat16 no near tie of a router on the way)
+    rep = Replayer(folders[(name, dtype)], dtype, 384, max_requests=4)
     steps = [{"entries": [("a", toks[:30], [29])], "end": []}]
     steps += [{"entries": [("a", toks[i:i + 1], [0])], "end": ["a"] if i == 329 else []} for i in range(30, 330)]
     got = tu.run(rep, steps)
     assert rep.engine.graph_replays > 250
-    want = plain_logits(folders[("D", dtype)], toks)
-    compare(got, {("a", i): want[i] for i in range(29, 330)}, dtype, f"long decoding {dtype}")
+    margins = []
+    want = plain_logits(folders[(name, dtype)], toks, margins)
+    compare(got, {("a", i): want[i] for i in range(29, 330)}, dtype, f"long decoding {dtype}",
+            {("a", i): m for i, m in enumerate(margins)})
 
 
 def test_a_far_token_shows_through_attention_alone(folders):
