@@ -226,12 +226,15 @@ __global__ __launch_bounds__(kScanWaves * 64) void linear_scan_kernel(
     const float* qp = q + row * ldq + (int64_t)g * D + d0;
     const float* ap = decay + row * ldd + (decay_per_head ? (int64_t)h : (int64_t)h * D + d0);
     const int astep = decay_per_head ? 0 : 1;
-    if (!decay_per_head && DPT % 4 == 0 && D == DPT * kScanParts && (((uintptr_t)kp | (uintptr_t)qp | (uintptr_t)ap) & 15) == 0) {
+    if (DPT % 4 == 0 && D == DPT * kScanParts &&
+        (((uintptr_t)kp | (uintptr_t)qp | (decay_per_head ? (uintptr_t)0 : (uintptr_t)ap)) & 15) == 0) {
       typedef float f32x4_t __attribute__((ext_vector_type(4)));      // (sixteen bytes a load where the rows allow)
+      const float one_decay = decay_per_head ? ap[0] : 0.f;
 #pragma unroll
       for (int i = 0; i + 3 < DPT; i += 4) {
-        const f32x4_t kv = *reinterpret_cast<const f32x4_t*>(kp + i), qv = *reinterpret_cast<const f32x4_t*>(qp + i),
-                      av = *reinterpret_cast<const f32x4_t*>(ap + i);
+        const f32x4_t kv = *reinterpret_cast<const f32x4_t*>(kp + i), qv = *reinterpret_cast<const f32x4_t*>(qp + i);
+        f32x4_t av = {one_decay, one_decay, one_decay, one_decay};
+        if (!decay_per_head) av = *reinterpret_cast<const f32x4_t*>(ap + i);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           kk[i + j] = kv[j];
