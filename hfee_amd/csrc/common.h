@@ -103,6 +103,34 @@ template <typename T> __device__ __forceinline__ T from_float(float v);
 template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
 template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) { return float_to_bf16(v); }
 
+// Four neighbouring values as float32, one load or store of 16 (float32) or 8 (bfloat16) bytes; p is aligned to that.
+template <typename T>
+__device__ __forceinline__ void load4(float (&v)[4], const T* p);
+template <>
+__device__ __forceinline__ void load4<float>(float (&v)[4], const float* p) {
+  const float4 t = *reinterpret_cast<const float4*>(p);
+  v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+template <>
+__device__ __forceinline__ void load4<bf16_t>(float (&v)[4], const bf16_t* p) {
+  const uint2 t = *reinterpret_cast<const uint2*>(p);
+  v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+  v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+}
+template <typename TN>
+__device__ __forceinline__ void store4(TN* p, const float (&v)[4]);
+template <>
+__device__ __forceinline__ void store4<float>(float* p, const float (&v)[4]) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+template <>
+__device__ __forceinline__ void store4<bf16_t>(bf16_t* p, const float (&v)[4]) {
+  bf16_t h[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) h[i] = from_float<bf16_t>(v[i]);
+  *reinterpret_cast<uint2*>(p) = *reinterpret_cast<const uint2*>(h);
+}
+
 // The activation of a gated feed-forward's gate, as the entry points name it.  The SiLU
 // (/root/reference/internal/ggml/ops.go:159-165) is written out where it is used, in the
 // form that each kernel has been measured with; the others are here, in forms that cost

@@ -68,33 +68,6 @@ __global__ __launch_bounds__(256) void gated_norm_add_kernel(
 // the row at once (K groups of four of y, y2, the gate and x), keeps the gated values in registers between the
 // sum of squares and the addition, and the new row between the second sum and the following norm.  A row is
 // read once, and a step of a few rows is one wait for memory instead of one a loop turn.
-template <typename TG>
-__device__ __forceinline__ void load4(float (&v)[4], const TG* p);
-template <>
-__device__ __forceinline__ void load4<float>(float (&v)[4], const float* p) {
-  const float4 t = *reinterpret_cast<const float4*>(p);
-  v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-}
-template <>
-__device__ __forceinline__ void load4<bf16_t>(float (&v)[4], const bf16_t* p) {
-  const uint2 t = *reinterpret_cast<const uint2*>(p);
-  v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
-  v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
-}
-template <typename TN>
-__device__ __forceinline__ void store4(TN* p, const float (&v)[4]);
-template <>
-__device__ __forceinline__ void store4<float>(float* p, const float (&v)[4]) {
-  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
-}
-template <>
-__device__ __forceinline__ void store4<bf16_t>(bf16_t* p, const float (&v)[4]) {
-  bf16_t h[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) h[i] = from_float<bf16_t>(v[i]);
-  *reinterpret_cast<uint2*>(p) = *reinterpret_cast<const uint2*>(h);
-}
-
 template <typename TG, typename TN, int K>
 __global__ __launch_bounds__(256) void gated_norm_add_held_kernel(
     float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ y2, float a, float b,

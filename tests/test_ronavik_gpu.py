@@ -258,13 +258,14 @@ def test_state_space_recurrence_in_portions(H, G, N, V):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_convolution_with_biases_carries_its_inputs(dtype):
+@pytest.mark.parametrize("C", [10, 24])
+def test_convolution_with_biases_carries_its_inputs(dtype, C):
     """A bias on the inputs stands only where there is an input: before a sequence's start are zeros.  Portions
     shorter than the taps; the state holds the inputs with their bias."""
     from hfee_amd.kernels import ops
     dt = DT[dtype]
     g = torch.Generator().manual_seed(1)
-    C, K, T = 10, 4, 19
+    K, T = 4, 19
     x = torch.randn(T, C, generator=g).to(dt)
     taps, ib, ob = torch.randn(C, K, generator=g), torch.randn(C, generator=g), torch.randn(C, generator=g)
     biased = (x.float() + ib).to(dt).double()
