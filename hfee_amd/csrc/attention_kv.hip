@@ -374,6 +374,73 @@ HFEE_API int hfee_attention_kv_plain(void* out, int64_t ld_out, const void* q, i
   return 0;
 }
 
+namespace {
+
+// The same products in float32 on the matrix cores, for steps of many tokens: a workgroup takes one head,
+// 64 tokens and 128 outputs, a wave 64 x 32 of them as two tiles of `32x32x2` float32 products (full
+// float32 operands and sums; nothing is rounded to fewer bits).  The tokens' inputs pass LDS in chunks of 64
+// (rows one word longer than that, so that the 32 rows a wave reads lie in different banks), a wave reads its
+// weights straight from memory, 32 neighbouring outputs a row.  An output's sum runs over the inputs in a
+// fixed order whatever else the tile holds: a token's result does not depend on the tokens beside it.
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+constexpr int kHeadMatrixTokens = 64, kHeadMatrixOutputs = 128, kHeadMatrixInputs = 64;
+
+__global__ __launch_bounds__(256) void head_linear_f32_matrix_kernel(
+    float* __restrict__ out, int64_t ldo, int64_t out_head_stride, const float* __restrict__ x, int64_t ldx,
+    int64_t x_head_stride, const float* __restrict__ w, int n_in, int n_out, int tail, int n) {
+  __shared__ float xs[kHeadMatrixTokens][kHeadMatrixInputs + 1];
+  const int h = blockIdx.y, t0 = blockIdx.x * kHeadMatrixTokens, o0 = blockIdx.z * kHeadMatrixOutputs;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 31, half = lane >> 5;
+  const int o = o0 + wave * 32 + col;
+  const float* wh = w + (int64_t)h * n_in * n_out;
+  const float* xh = x + (int64_t)h * x_head_stride;
+  f32x16_t acc0, acc1;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc0[v] = acc1[v] = 0.f;
+  for (int k0 = 0; k0 < n_in; k0 += kHeadMatrixInputs) {
+    const int count = min(kHeadMatrixInputs, n_in - k0);
+    // a lane's weights of the chunk are asked for first, so that they travel while the inputs are put into LDS:
+    // of each pair of inputs lanes 0..31 take the first, lanes 32..63 the second
+    float b[kHeadMatrixInputs / 2];
+#pragma unroll
+    for (int p = 0; p < kHeadMatrixInputs / 2; ++p) {
+      const int k = 2 * p + half;
+      b[p] = k < count && o < n_out ? wh[(int64_t)(k0 + k) * n_out + o] : 0.f;
+    }
+    __syncthreads();                                   // (the chunk before has been read)
+    for (int e = threadIdx.x; e < kHeadMatrixTokens * kHeadMatrixInputs; e += 256) {
+      const int r = e / kHeadMatrixInputs, i = e - r * kHeadMatrixInputs;
+      xs[r][i] = t0 + r < n && k0 + i < n_in ? xh[(int64_t)(t0 + r) * ldx + k0 + i] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int p = 0; p < kHeadMatrixInputs / 2; ++p) {    // (beyond `count` both operands are zero)
+      const int k = 2 * p + half;
+      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(xs[col][k], b[p], acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(xs[32 + col][k], b[p], acc1, 0, 0, 0);
+    }
+  }
+  if (o < n_out) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {                      // a lane's sixteen sums: rows 8 (v / 4) + 4 half + v % 4 of its column
+      const int r = t0 + (v >> 2) * 8 + half * 4 + (v & 3);
+      if (r < n) out[(int64_t)r * ldo + (int64_t)h * out_head_stride + o] = acc0[v];
+      if (r + 32 < n) out[(int64_t)(r + 32) * ldo + (int64_t)h * out_head_stride + o] = acc1[v];
+    }
+  }
+  if (blockIdx.z == 0) {
+    const int count = min(kHeadMatrixTokens, n - t0);
+    for (int e = threadIdx.x; e < count * tail; e += blockDim.x) {
+      const int r = e / tail, i = e - r * tail;
+      out[(int64_t)(t0 + r) * ldo + (int64_t)h * out_head_stride + n_out + i] =
+          x[(int64_t)(t0 + r) * ldx + (int64_t)h * x_head_stride + n_in + i];
+    }
+  }
+}
+
+}  // namespace
+
 HFEE_API int hfee_head_linear(void* out, int64_t ldo, int64_t out_head_stride, const void* x, int64_t ldx,
                               int64_t x_head_stride, const void* w, int dtype, int heads, int n_in, int n_out,
                               int tail, int n, hipStream_t stream) {
@@ -384,7 +451,11 @@ HFEE_API int hfee_head_linear(void* out, int64_t ldo, int64_t out_head_stride, c
   HFEE_REQUIRE((n_out + kHeadLinearOutputs - 1) / kHeadLinearOutputs <= 65535, "head_linear: too many outputs a head");
   dim3 grid((n + kHeadLinearTokens - 1) / kHeadLinearTokens, heads, (n_out + kHeadLinearOutputs - 1) / kHeadLinearOutputs);
   const size_t lds = ((size_t)kHeadLinearTokens * n_in + kHeadLinearSlices * kHeadLinearTokens * kHeadLinearOutputs) * sizeof(float);
-  if (dtype == 0)
+  if (dtype == 0 && n >= 32) {       // (out == x with a tail would be read and written by different workgroups: never so)
+    dim3 tiles((n + kHeadMatrixTokens - 1) / kHeadMatrixTokens, heads, (n_out + kHeadMatrixOutputs - 1) / kHeadMatrixOutputs);
+    head_linear_f32_matrix_kernel<<<tiles, 256, 0, stream>>>((float*)out, ldo, out_head_stride, (const float*)x, ldx,
+        x_head_stride, (const float*)w, n_in, n_out, tail, n);
+  } else if (dtype == 0)
     head_linear_kernel<float><<<grid, 256, lds, stream>>>((float*)out, ldo, out_head_stride, (const float*)x, ldx,
         x_head_stride, (const float*)w, n_in, n_out, tail, n);
   else if (dtype == 1)

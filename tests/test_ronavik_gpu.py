@@ -211,6 +211,29 @@ def test_recurrent_unit_in_portions(dtype, W, blocks):
     assert bool(torch.isnan(state[1]).all()) and float(state[2].abs().sum()) == 0.0
 
 
+@pytest.mark.parametrize("n", [5, 33, 150])
+def test_products_a_block_in_32_bit(n):
+    """out[t, h] = W_h^T x[t, h] with what lies behind a head's inputs copied behind its outputs: a few tokens
+    on the vector units, many on the matrix cores in float32 (tiles of 64 tokens and 128 outputs that the
+    sizes do not fill, inputs that are no whole chunk); a token's result does not depend on its company."""
+    from hfee_amd.kernels import ops
+    g = torch.Generator().manual_seed(n)
+    heads, n_in, n_out, tail = 3, 70, 150, 5
+    x = torch.randn(n, heads * (n_in + tail) + 3, generator=g)
+    w = torch.randn(heads, n_in, n_out, generator=g)
+    out = torch.full((n, heads * (n_out + tail) + 2), float("nan"), device="cuda")
+    ops.head_linear(out, x.cuda(), w.cuda(), heads, n_in, n_out, tail=tail)
+    xh = x[:, :heads * (n_in + tail)].view(n, heads, n_in + tail).double()
+    want = torch.cat([torch.einsum("thi,hio->tho", xh[:, :, :n_in], w.double()), xh[:, :, n_in:]], dim=2).reshape(n, -1)
+    got = out.cpu()
+    assert ru.rel(got[:, :want.shape[1]], want) < 2e-6
+    assert bool(torch.isnan(got[:, want.shape[1]:]).all())
+    if n >= 64:          # the first tokens alone, in a step of their own size: the same bits
+        alone = torch.zeros(40, out.shape[1], device="cuda")
+        ops.head_linear(alone, x[:40].cuda(), w.cuda(), heads, n_in, n_out, tail=tail)
+        assert torch.equal(alone.cpu()[:, :want.shape[1]], got[:40, :want.shape[1]])
+
+
 @pytest.mark.parametrize("H,G,N,V", [(4, 2, 16, 8), (3, 1, 10, 12), (2, 2, 33, 70), (8, 4, 64, 32)])
 def test_state_space_recurrence_in_portions(H, G, N, V):
     """S <- a S + dt B x^T with one decay a head, y = S^T C, by its definition in float64 against the kernel
