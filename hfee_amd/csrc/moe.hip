@@ -325,6 +325,144 @@ __global__ __launch_bounds__(256) void moe_group_down_kernel(float* __restrict__
   }
 }
 
+// The grouped products through LDS.  A workgroup takes a tile of up to 64 pairs of one expert and 256 rows of
+// weights (KIND 0: 128 rows of the gate's matrix and the same 128 of the up matrix); K in steps of 32: every
+// thread asks for its 16-byte pieces of the next step (one of the pairs' rows, four of the weights') while the
+// matrix cores work on the current one out of LDS, then lays them into the other buffer; rows of 40 elements
+// so that the operand reads of 32 rows spread over the banks.  A wave owns 64 weight rows (KIND 0: 32 of each
+// matrix) x 64 pairs as 2 x 2 tiles of `32x32x16`, the weights as the row operand, so that a lane ends with
+// four neighbouring rows of the matrix for one pair and stores them at once.  A sum runs over K in the same
+// order whichever pairs share the tile.
+//   KIND 0: act = silu(gate) * up      KIND 1: act = relu(weight * up)^2      KIND 2: out (+)= scale * down
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+constexpr int kStageK = 32, kStagePitch = 40;
+
+template <int KIND>
+__global__ __launch_bounds__(256) void moe_group_tiled_kernel(
+    void* __restrict__ dst, int64_t ldo, const bf16_t* __restrict__ src, int64_t lds_rows, const bf16_t* __restrict__ w0,
+    const bf16_t* __restrict__ w1, const int* __restrict__ order, const int* __restrict__ tiles, int most_tiles, int top,
+    int n_rows, int K, int add, const float* __restrict__ pair_weights, float weight) {
+  __shared__ __attribute__((aligned(16))) bf16_t As[2][kTilePairs * kStagePitch];
+  __shared__ __attribute__((aligned(16))) bf16_t Ws[2][kTileRows * kStagePitch];
+  if ((int)blockIdx.x >= tiles[3 * most_tiles]) return;
+  const int* tl = tiles + 3 * blockIdx.x;
+  const int e = tl[0], first = tl[1], count = tl[2];
+  constexpr int kRowsOut = KIND == 0 ? kTileRows / 2 : kTileRows;      // rows of the result a workgroup makes
+  const int row0 = blockIdx.y * kRowsOut;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+  // what this thread brings of every step: piece (tid & 3) of pair row tid / 4, and of weight rows tid / 4 + 64 p
+  const int piece = (tid & 3) * 8, srow = tid >> 2;
+  const int my_pair = order[first + (srow < count ? srow : 0)];
+  const bf16_t* a_src = src + (int64_t)(KIND == 2 ? my_pair : my_pair / top) * lds_rows + piece;
+  const bf16_t* w_src[4];
+  bool w_ok[4];
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    const int s = srow + 64 * p;                                        // the row's place in the staged tile
+    const bf16_t* base = KIND == 0 && s >= kRowsOut ? w1 : w0;
+    const int row = row0 + (KIND == 0 && s >= kRowsOut ? s - kRowsOut : s);
+    w_ok[p] = row < n_rows;
+    w_src[p] = base + ((int64_t)e * n_rows + (w_ok[p] ? row : 0)) * K + piece;
+  }
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  u32x4 ra = *reinterpret_cast<const u32x4*>(a_src), rw[4];
+#pragma unroll
+  for (int p = 0; p < 4; ++p) rw[p] = w_ok[p] ? *reinterpret_cast<const u32x4*>(w_src[p]) : zero;
+  *reinterpret_cast<u32x4*>(&As[0][srow * kStagePitch + piece]) = ra;
+#pragma unroll
+  for (int p = 0; p < 4; ++p) *reinterpret_cast<u32x4*>(&Ws[0][(srow + 64 * p) * kStagePitch + piece]) = rw[p];
+  __syncthreads();
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  const int lrow = lane & 31, lk = (lane >> 5) * 8;
+  // the wave's two groups of 32 staged weight rows
+  const int base_i[2] = {KIND == 0 ? wave * 32 : wave * 64, KIND == 0 ? kRowsOut + wave * 32 : wave * 64 + 32};
+  const int steps = K / kStageK;
+  int buf = 0;
+  for (int kt = 0; kt < steps; ++kt) {
+    if (kt + 1 < steps) {
+      const int k = (kt + 1) * kStageK;
+      ra = *reinterpret_cast<const u32x4*>(a_src + k);
+#pragma unroll
+      for (int p = 0; p < 4; ++p) rw[p] = w_ok[p] ? *reinterpret_cast<const u32x4*>(w_src[p] + k) : zero;
+    }
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      bf16x8 a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        a[i] = *reinterpret_cast<const bf16x8*>(&Ws[buf][(base_i[i] + lrow) * kStagePitch + ks * 16 + lk]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        b[j] = *reinterpret_cast<const bf16x8*>(&As[buf][(j * 32 + lrow) * kStagePitch + ks * 16 + lk]);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < steps) {
+      *reinterpret_cast<u32x4*>(&As[buf ^ 1][srow * kStagePitch + piece]) = ra;
+#pragma unroll
+      for (int p = 0; p < 4; ++p) *reinterpret_cast<u32x4*>(&Ws[buf ^ 1][(srow + 64 * p) * kStagePitch + piece]) = rw[p];
+    }
+    __syncthreads();
+    buf ^= 1;
+  }
+
+  // register r of lane l in tile (i, j): row 8 (r / 4) + 4 (l / 32) + r % 4 of the wave's group i, pair 32 j + l % 32
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int at = j * 32 + lrow;
+    if (at >= count) continue;
+    const int pair = order[first + at];
+    if constexpr (KIND == 0) {
+      bf16_t* o = (bf16_t*)dst + (int64_t)pair * ldo;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int f = row0 + wave * 32 + 8 * q + 4 * (lane >> 5);
+        if (f >= n_rows) continue;
+        bf16_t four[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float g = acc[0][j][4 * q + r];
+          four[r] = float_to_bf16(g / (1.0f + expf(-g)) * acc[1][j][4 * q + r]);
+        }
+        *reinterpret_cast<u32x2*>(o + f) = *reinterpret_cast<const u32x2*>(four);
+      }
+    } else {
+      const float scale = KIND == 1 ? (pair_weights != nullptr ? pair_weights[pair] : 1.0f)
+                                    : add ? (pair_weights != nullptr ? pair_weights[pair] : weight) : 1.0f;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int f = row0 + wave * 64 + 32 * i + 8 * q + 4 * (lane >> 5);
+          if (f >= n_rows) continue;
+          if constexpr (KIND == 1) {
+            bf16_t four[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const float u = fmaxf(acc[i][j][4 * q + r] * scale, 0.f);
+              four[r] = float_to_bf16(u * u);
+            }
+            *reinterpret_cast<u32x2*>((bf16_t*)dst + (int64_t)pair * ldo + f) = *reinterpret_cast<const u32x2*>(four);
+          } else {
+            float* o = (float*)dst + (int64_t)pair * ldo + f;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[r] = add ? fmaf(acc[i][j][4 * q + r], scale, o[r]) : acc[i][j][4 * q + r];
+          }
+        }
+    }
+  }
+}
+
 // x[t] += sum_j weight_tj y[t * top + j], j ascending.
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x, int64_t ldx, const float* __restrict__ y,
                                                           const float* __restrict__ pair_weights, float weight, int top,
@@ -407,16 +545,18 @@ HFEE_API int hfee_moe_grouped(float* x, int64_t ldx, const void* h, int64_t ldh,
   const int most = hfee_moe_group_tiles(n, top, experts);
   moe_group_kernel<<<1, 1024, 4 * experts * sizeof(int), stream>>>(order, tiles, most, chosen, table, token_ids, n, top, experts);
   HFEE_CHECK_LAUNCH("moe_group");
+  // (rows in whole groups of four: ff and width are multiples of 32)
   if (w_gate != nullptr)
-    moe_group_up_kernel<0><<<dim3(most, (ff + kTileRows - 1) / kTileRows), 256, 0, stream>>>(
-        (bf16_t*)act, (const bf16_t*)h, ldh, (const bf16_t*)w_gate, (const bf16_t*)w_up, order, tiles, most, top, ff, width, nullptr);
+    moe_group_tiled_kernel<0><<<dim3(most, (ff + kTileRows / 2 - 1) / (kTileRows / 2)), 256, 0, stream>>>(
+        act, ff, (const bf16_t*)h, ldh, (const bf16_t*)w_gate, (const bf16_t*)w_up, order, tiles, most, top, ff, width, 0,
+        nullptr, 1.0f);
   else
-    moe_group_up_kernel<1><<<dim3(most, (ff + kTileRows - 1) / kTileRows), 256, 0, stream>>>(
-        (bf16_t*)act, (const bf16_t*)h, ldh, nullptr, (const bf16_t*)w_up, order, tiles, most, top, ff, width, in_weights);
+    moe_group_tiled_kernel<1><<<dim3(most, (ff + kTileRows - 1) / kTileRows), 256, 0, stream>>>(
+        act, ff, (const bf16_t*)h, ldh, (const bf16_t*)w_up, nullptr, order, tiles, most, top, ff, width, 0, in_weights, 1.0f);
   HFEE_CHECK_LAUNCH("moe_group_up");
-  moe_group_down_kernel<<<dim3(most, (width + kTileRows - 1) / kTileRows), 256, 0, stream>>>(
-      top == 1 ? x : y, top == 1 ? ldx : (int64_t)width, (const bf16_t*)act, (const bf16_t*)w_down, order, tiles, most, ff, width,
-      top == 1 ? 1 : 0, pair_weights, weight);
+  moe_group_tiled_kernel<2><<<dim3(most, (width + kTileRows - 1) / kTileRows), 256, 0, stream>>>(
+      top == 1 ? (void*)x : (void*)y, top == 1 ? ldx : (int64_t)width, (const bf16_t*)act, ff, (const bf16_t*)w_down, nullptr,
+      order, tiles, most, top, width, ff, top == 1 ? 1 : 0, pair_weights, weight);
   HFEE_CHECK_LAUNCH("moe_group_down");
   if (top > 1) {
     int parts = (width + 255) / 256;
