@@ -20,11 +20,11 @@
 // fixed order; every token reads the rows of its own experts.  For steps of few tokens, whose time is
 // the experts' bytes, and for float32.
 //
-// Grouped (moe_group, moe_group_up, moe_group_down, moe_combine; bfloat16): the (token, expert) pairs of a
-// step are put in the order of their experts on the device, cut into tiles of 64 pairs of one expert, and
-// a workgroup multiplies a tile by 256 rows of that expert's matrix on the matrix cores (a wave 64 x 64
-// of v_mfma_f32_16x16x32_bf16, operands straight from memory): an expert's matrices are read once a
-// 64 pairs and not once a pair.  A pair's numbers do not depend on which pairs share its tile.
+// Grouped (moe_group, moe_group_tiled, moe_combine; bfloat16): the (token, expert) pairs of a step are put
+// in the order of their experts on the device, cut into tiles of 64 pairs of one expert, and a workgroup
+// multiplies a tile by 256 rows of that expert's matrix on the matrix cores (both operands staged through
+// LDS in steps of 32 columns, a wave 64 x 64 of v_mfma_f32_32x32x16_bf16): an expert's matrices are read
+// once a 64 pairs and not once a pair.  A pair's numbers do not depend on which pairs share its tile.
 #include "common.h"
 
 using namespace hfee;
@@ -142,14 +142,8 @@ __global__ __launch_bounds__(256) void moe_down_kernel(float* __restrict__ x, in
 
 // ---------------------------------------------------------------------------- grouped
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-
-union Operand {
-  u32x4 u;
-  bf16x8 v;
-};
 
 constexpr int kTilePairs = 64, kTileRows = 256;
 
@@ -194,135 +188,6 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(int* __restrict__ order
       tl[1] = starts[e] + i * kTilePairs;
       tl[2] = min(kTilePairs, counts[e] - i * kTilePairs);
     }
-}
-
-// C[64 pairs][64 rows of B] (+)= A B^T for one wave: A rows through a_rows (pointers to the K elements of
-// each of the lane's four pair rows), B rows from b (row stride K; rows at and beyond n_rows read row 0).
-template <int NB>
-__device__ __forceinline__ void tile_products(f32x4 (&acc)[NB][4][4], const bf16_t* const (&a_rows)[4],
-                                              const bf16_t* const (&b)[NB], int64_t K, int row0, int n_rows, int lane) {
-  const int r16 = lane & 15, kg = (lane >> 4) * 8;
-  const bf16_t* b_rows[NB][4];
-#pragma unroll
-  for (int m = 0; m < NB; ++m)
-#pragma unroll
-    for (int nt = 0; nt < 4; ++nt) {
-      const int row = row0 + nt * 16 + r16;
-      b_rows[m][nt] = b[m] + (int64_t)(row < n_rows ? row : 0) * K + kg;
-    }
-  for (int64_t k0 = 0; k0 < K; k0 += 32) {
-    Operand a[4], w[NB][4];
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt) a[mt].u = *reinterpret_cast<const u32x4*>(a_rows[mt] + k0 + kg);
-#pragma unroll
-    for (int m = 0; m < NB; ++m)
-#pragma unroll
-      for (int nt = 0; nt < 4; ++nt) w[m][nt].u = *reinterpret_cast<const u32x4*>(b_rows[m][nt] + k0);
-#pragma unroll
-    for (int m = 0; m < NB; ++m)
-#pragma unroll
-      for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
-          acc[m][nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[m][nt].v, a[mt].v, acc[m][nt][mt], 0, 0, 0);
-  }
-}
-
-template <int FORM>
-__global__ __launch_bounds__(256) void moe_group_up_kernel(bf16_t* __restrict__ act, const bf16_t* __restrict__ h, int64_t ldh,
-                                                           const bf16_t* __restrict__ w_gate, const bf16_t* __restrict__ w_up,
-                                                           const int* __restrict__ order, const int* __restrict__ tiles,
-                                                           int most_tiles, int top, int F, int width,
-                                                           const float* __restrict__ in_weights) {
-  if ((int)blockIdx.x >= tiles[3 * most_tiles]) return;
-  const int* tl = tiles + 3 * blockIdx.x;
-  const int e = tl[0], first = tl[1], count = tl[2];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r16 = lane & 15;
-  const int row0 = blockIdx.y * kTileRows + wave * 64;
-  if (row0 >= F) return;
-  int pair[4];
-  const bf16_t* a_rows[4];
-#pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
-    const int r = mt * 16 + r16;
-    pair[mt] = order[first + (r < count ? r : 0)];
-    a_rows[mt] = h + (int64_t)(pair[mt] / top) * ldh;
-  }
-  if constexpr (FORM == 1) {      // no gate: the square of relu, the pair's weight on the sum
-    const bf16_t* const b1[1] = {w_up + (int64_t)e * F * width};
-    f32x4 acc1[1][4][4] = {};
-    tile_products<1>(acc1, a_rows, b1, width, row0, F, lane);
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
-      if (mt * 16 + r16 >= count) continue;
-      const float wt = in_weights != nullptr ? in_weights[pair[mt]] : 1.0f;
-#pragma unroll
-      for (int nt = 0; nt < 4; ++nt) {
-        const int f = row0 + nt * 16 + (lane >> 4) * 4;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float u = fmaxf(acc1[0][nt][mt][i] * wt, 0.f);
-          if (f + i < F) act[(int64_t)pair[mt] * F + f + i] = float_to_bf16(u * u);
-        }
-      }
-    }
-    return;
-  }
-  const bf16_t* const b[2] = {w_gate + (int64_t)e * F * width, w_up + (int64_t)e * F * width};
-  f32x4 acc[2][4][4] = {};
-  tile_products<2>(acc, a_rows, b, width, row0, F, lane);
-  // register i of lane l: row of the matrix 16 nt + 4 (l / 16) + i, pair row 16 mt + l % 16
-#pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
-    if (mt * 16 + r16 >= count) continue;
-#pragma unroll
-    for (int nt = 0; nt < 4; ++nt) {
-      const int f = row0 + nt * 16 + (lane >> 4) * 4;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float g = acc[0][nt][mt][i];
-        if (f + i < F) act[(int64_t)pair[mt] * F + f + i] = float_to_bf16(g / (1.0f + expf(-g)) * acc[1][nt][mt][i]);
-      }
-    }
-  }
-}
-
-// out: x (float32 [n, width]) when a token has one expert (then out[t] += weight * product), else
-// y (float32 [pairs, width]) = product.
-__global__ __launch_bounds__(256) void moe_group_down_kernel(float* __restrict__ out, int64_t ldo, const bf16_t* __restrict__ act,
-                                                             const bf16_t* __restrict__ w_down, const int* __restrict__ order,
-                                                             const int* __restrict__ tiles, int most_tiles, int F, int width,
-                                                             int add, const float* __restrict__ pair_weights, float weight) {
-  if ((int)blockIdx.x >= tiles[3 * most_tiles]) return;
-  const int* tl = tiles + 3 * blockIdx.x;
-  const int e = tl[0], first = tl[1], count = tl[2];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r16 = lane & 15;
-  const int row0 = blockIdx.y * kTileRows + wave * 64;
-  if (row0 >= width) return;
-  int pair[4];
-  const bf16_t* a_rows[4];
-#pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
-    const int r = mt * 16 + r16;
-    pair[mt] = order[first + (r < count ? r : 0)];
-    a_rows[mt] = act + (int64_t)pair[mt] * F;
-  }
-  const bf16_t* const b[1] = {w_down + (int64_t)e * width * F};
-  f32x4 acc[1][4][4] = {};
-  tile_products<1>(acc, a_rows, b, F, row0, width, lane);
-#pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
-    if (mt * 16 + r16 >= count) continue;
-    const float scale = add ? (pair_weights != nullptr ? pair_weights[pair[mt]] : weight) : 1.0f;
-#pragma unroll
-    for (int nt = 0; nt < 4; ++nt) {
-      const int c = row0 + nt * 16 + (lane >> 4) * 4;
-      float* o = out + (int64_t)pair[mt] * ldo + c;
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (c + i < width) o[i] = add ? fmaf(acc[0][nt][mt][i], scale, o[i]) : acc[0][nt][mt][i];
-    }
-  }
 }
 
 // The grouped products through LDS.  A workgroup takes a tile of up to 64 pairs of one expert and 256 rows of
