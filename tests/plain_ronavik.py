@@ -117,8 +117,10 @@ def routed_experts(h, w, pre, mlp, margins=None):
     logits' spread over the experts (infinite where every expert is chosen)."""
     E, top = mlp["router"]["experts"], mlp["router"]["top"]
     z = h @ w[pre + "router"].T
-    s = torch.sigmoid(z)
-    vals, idx = torch.topk(s, top, dim=-1)
+    # (the largest scores are the largest logits; chosen by the logits, so that two scores that both round
+    # to one cannot tie)
+    idx = torch.topk(z, top, dim=-1).indices
+    vals = torch.sigmoid(torch.gather(z, -1, idx))
     if margins is not None:
         if top < E:
             best = torch.topk(z, top + 1, dim=-1).values
