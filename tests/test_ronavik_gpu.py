@@ -573,7 +573,7 @@ def greedy(folder, prompt, count):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_greedy_generation_through_the_entry_point(folders, dtype):
     from hfee_amd import LLM, SamplingParams
-    folder = folders[("A", dtype)]
+    folder = folders[("A" if dtype == "float32" else "A every expert", dtype)]      # (no router's near tie in bfloat16)
     llm = LLM(folder, dtype=dtype, num_ctx=128, num_parallel=3, max_batch_tokens=24)
     g = np.random.default_rng(5)
     prompts = [g.integers(0, 131, size=n).tolist() for n in (5, 40, 1, 17, 33)]
