@@ -5,5 +5,6 @@ from .llama import LlamaConfig, RopeScaling
 from .vofezen import VofezenConfig
 from .sabezen import SabezenConfig
 from .ronavik import RonavikConfig
+from .saposun import SaposunConfig
 from .registry import (register_architecture, lookup_architecture, architecture_of,
                        architecture_names, config_from_dict, config_from_folder, model_spec_of)

@@ -32,7 +32,9 @@ struct KvLayout {
   }
 };
 
-inline int make_kv_layout(KvLayout* out, int kv_heads, int dk, int dv, int page_size) {
+// A page may hold `sections` such parts a head, one behind the other: the tokens' keys and values first,
+// then (a second section) one pooled key and value for every block of tokens, under the block's number.
+inline int make_kv_layout(KvLayout* out, int kv_heads, int dk, int dv, int page_size, int sections = 1) {
   if (page_size < 16 || (page_size & (page_size - 1)) != 0)
     return fail("page_size must be a power of two >= 16, got %d", page_size);
   if (kv_heads < 1 || dk < 1 || dv < 1) return fail("bad cache shape: kv_heads %d dk %d dv %d", kv_heads, dk, dv);
@@ -40,11 +42,38 @@ inline int make_kv_layout(KvLayout* out, int kv_heads, int dk, int dv, int page_
   out->dk = dk;
   out->dv = dv;
   out->page_size = page_size;
-  out->head_stride = (int64_t)page_size * (dk + dv);
+  if (sections < 1 || sections > 2) return fail("a page holds one or two sections a head, not %d", sections);
+  out->head_stride = (int64_t)sections * page_size * (dk + dv);
   out->page_stride = (int64_t)kv_heads * out->head_stride;
   int s = 0;
   while ((1 << s) < page_size) ++s;
   out->page_shift = s;
+  return 0;
+}
+
+// What a query at position p sees: the keys first_key(p) .. p, and the pooled blocks 0 .. pooled_blocks(p) - 1
+// (block b holds the positions b * pool .. b * pool + pool - 1 and is seen once all of them have left the
+// window: b * pool + pool - 1 <= p - window).
+struct KeySight {
+  int window;            // 0: every earlier position
+  int pool;              // 0: no pooled blocks
+  float softcap;         // 0: scores as they are
+  int64_t pool_offset;   // elements from a (page, head)'s first section to its pooled one
+
+  __host__ __device__ __forceinline__ int first_key(int p) const { return window > 0 && p - window + 1 > 0 ? p - window + 1 : 0; }
+  __host__ __device__ __forceinline__ int pooled_blocks(int p) const {
+    return pool > 0 && window > 0 && p - window + 1 >= pool ? (p - window + 1) / pool : 0;
+  }
+  __device__ __forceinline__ float capped(float s) const { return softcap > 0.f ? softcap * tanhf(s / softcap) : s; }
+};
+
+inline int make_key_sight(KeySight* out, int window, int pool, float softcap, int sections, int page_size, int dk, int dv) {
+  if (window < 0 || pool < 0 || !(softcap >= 0.f)) return fail("bad window %d, pool %d or softcap %f", window, pool, (double)softcap);
+  if (pool > 0 && sections != 2) return fail("pooled blocks live in a page's second section");
+  out->window = window;
+  out->pool = pool;
+  out->softcap = softcap;
+  out->pool_offset = (int64_t)page_size * (dk + dv);
   return 0;
 }
 

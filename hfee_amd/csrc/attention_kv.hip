@@ -134,18 +134,107 @@ __global__ __launch_bounds__(256) void qk_norm_write_kernel(
   for (int d = lane; d < lay.dv; d += 64) cache[lay.value_offset(page, g, slot, d)] = finite_for_cache<T>(p[d]);
 }
 
+// ---------------------------------------------------------------- rotation + value norm + cache write, from float32
+// One wave a (token, unit), for projections that arrive in float32 (behind a short convolution): the
+// units of a token are its query heads (rotated, written to q_out in the cache's dtype), its key heads
+// (rotated into the token's slot) and its value heads (divided by their root mean square over the head
+// where value_eps >= 0, into the slot).  The first 2 * half dims of a q or k head are rotated, pairs
+// (i, i + half); cos/sin tables [positions][half].
+template <typename T>
+__global__ __launch_bounds__(256) void rotate_norm_write_kernel(
+    T* __restrict__ q_out, int64_t ldqo, const float* __restrict__ q, int64_t ldq, int num_heads,
+    const float* __restrict__ k, int64_t ldk, const float* __restrict__ v, int64_t ldv, float value_eps,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t, int half,
+    const int* __restrict__ positions, const int* __restrict__ token_segment, const int* __restrict__ block_tables,
+    int bt_stride, T* __restrict__ cache, KvLayout lay, int n) {
+  const int units = num_heads + (k != nullptr ? 2 * lay.kv_heads : 0);
+  const int64_t item = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (item >= (int64_t)n * units) return;
+  const int t = (int)(item / units), unit = (int)(item % units), lane = threadIdx.x & 63;
+  const int pos = positions[t];
+  const float* c = cos_t + (int64_t)pos * half;
+  const float* s = sin_t + (int64_t)pos * half;
+  auto turned = [&](const float* p, int d) {
+    if (d < half) return p[d] * c[d] - p[d + half] * s[d];
+    if (d < 2 * half) return p[d] * c[d - half] + p[d - half] * s[d - half];
+    return p[d];
+  };
+  if (unit < num_heads) {
+    const float* p = q + (int64_t)t * ldq + (int64_t)unit * lay.dk;
+    T* o = q_out + (int64_t)t * ldqo + (int64_t)unit * lay.dk;
+    for (int d = lane; d < lay.dk; d += 64) o[d] = from_float<T>(turned(p, d));
+    return;
+  }
+  const int page = block_tables[(int64_t)token_segment[t] * bt_stride + (pos >> lay.page_shift)];
+  const int slot = pos & (lay.page_size - 1);
+  if (unit < num_heads + lay.kv_heads) {
+    const int g = unit - num_heads;
+    const float* p = k + (int64_t)t * ldk + (int64_t)g * lay.dk;
+    for (int d = lane; d < lay.dk; d += 64)
+      cache[lay.key_offset(page, g, slot, d)] = finite_for_cache<T>(from_float<T>(turned(p, d)));
+    return;
+  }
+  const int g = unit - num_heads - lay.kv_heads;
+  const float* p = v + (int64_t)t * ldv + (int64_t)g * lay.dv;
+  float inv = 1.0f;
+  if (value_eps >= 0.f) {
+    float ss = 0.f;
+    for (int d = lane; d < lay.dv; d += 64) ss = fmaf(p[d], p[d], ss);
+    inv = 1.0f / sqrtf(wave_sum(ss) / (float)lay.dv + value_eps);
+  }
+  for (int d = lane; d < lay.dv; d += 64)
+    cache[lay.value_offset(page, g, slot, d)] = finite_for_cache<T>(from_float<T>(p[d] * inv));
+}
+
+// ---------------------------------------------------------------- pooled blocks
+// One wave a (token, key/value head): a token at the last position of a block of `pool` positions
+// (position % pool == pool - 1) leaves the block's key and value in the pooled section under the
+// block's number: the means of the block's keys and values as the cache holds them, summed in the
+// order of the positions in float32.  Every other token's wave has nothing to do.  Runs behind the
+// launch that wrote the step's keys and values.
+template <typename T>
+__global__ __launch_bounds__(256) void kv_pool_write_kernel(
+    T* __restrict__ cache, KvLayout lay, int pool, int64_t pool_offset, const int* __restrict__ positions,
+    const int* __restrict__ token_segment, const int* __restrict__ block_tables, int bt_stride, int n) {
+  const int64_t item = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (item >= (int64_t)n * lay.kv_heads) return;
+  const int t = (int)(item / lay.kv_heads), g = (int)(item % lay.kv_heads), lane = threadIdx.x & 63;
+  const int pos = positions[t];
+  if (pos % pool != pool - 1) return;
+  const int b = pos / pool;
+  const int* bt = block_tables + (int64_t)token_segment[t] * bt_stride;
+  T* pooled = cache + pool_offset;
+  const int to_page = bt[b >> lay.page_shift], to_slot = b & (lay.page_size - 1);
+  const float share = 1.0f / (float)pool;
+  for (int d = lane; d < lay.dk + lay.dv; d += 64) {
+    float sum = 0.f;
+    for (int j = pos - pool + 1; j <= pos; ++j) {
+      const int page = bt[j >> lay.page_shift], slot = j & (lay.page_size - 1);
+      sum += to_float<T>(cache[d < lay.dk ? lay.key_offset(page, g, slot, d) : lay.value_offset(page, g, slot, d - lay.dk)]);
+    }
+    pooled[d < lay.dk ? lay.key_offset(to_page, g, to_slot, d) : lay.value_offset(to_page, g, to_slot, d - lay.dk)] =
+        from_float<T>(sum * share);
+  }
+}
+
 // ---------------------------------------------------------------- plain attention
 // Lane (j mod 64) owns key j, so which lane adds which term depends only on the key's
 // absolute position: a token's result does not change with the way the work was cut into
 // steps, with the batch around it or with page numbers.
 constexpr int kMaxDvPerLane = 16;     // value sizes up to 1,024
 
+// What a query sees besides the keys up to its own position (`KeySight`): with a window it sees the last
+// `window` positions, itself included; with pooled blocks it also sees, for every block of `pool`
+// positions that lies wholly before the window, one key and one value (the block's means, kept in the
+// pooled section of the cache under the block's number); a score may be capped as
+// cap * tanh(score / cap) before it is weighed.  Tokens and blocks share one softmax.
 template <typename T>
 __global__ __launch_bounds__(64) void attention_kv_plain_kernel(
     T* __restrict__ out, int64_t ld_out, const T* __restrict__ q, int64_t ldq,
     const T* __restrict__ cache, KvLayout lay, const int* __restrict__ positions,
     const int* __restrict__ token_segment, const int* __restrict__ block_tables, int bt_stride,
-    int num_heads, float scale, const float* __restrict__ sinks, int weighting) {
+    int num_heads, float scale, const float* __restrict__ sinks, int weighting, KeySight sight,
+    const T* __restrict__ gate, int64_t ld_gate) {
   extern __shared__ float lds[];
   const int dk = lay.dk, dv = lay.dv;
   float* qs = lds;            // [dk]
@@ -154,18 +243,26 @@ __global__ __launch_bounds__(64) void attention_kv_plain_kernel(
   const int kvh = h / (num_heads / lay.kv_heads);
   const int pos = positions[t];
   const int* bt = block_tables + (int64_t)token_segment[t] * bt_stride;
+  const int first = sight.first_key(pos), blocks = sight.pooled_blocks(pos);
+  const T* pooled = cache + sight.pool_offset;
 
   for (int d = lane; d < dk; d += 64) qs[d] = to_float<T>(q[(int64_t)t * ldq + (int64_t)h * dk + d]);
   __syncthreads();
 
+  // the score of entry j of a section (the tokens' or the pooled blocks'), as the softmax takes it
+  auto score = [&](const T* section, int j) {
+    const T* kr = section + lay.key_offset(bt[j >> lay.page_shift], kvh, j & (lay.page_size - 1), 0);
+    float s = 0.f;
+    for (int d = 0; d < dk; ++d) s = fmaf(qs[d], to_float<T>(kr[d]), s);
+    return sight.capped(s * scale);
+  };
   float m = -INFINITY;
-  for (int base = 0; weighting == 0 && base <= pos; base += 64) {
-    const int j = base + lane;
-    if (j <= pos) {
-      const T* kr = cache + lay.key_offset(bt[j >> lay.page_shift], kvh, j & (lay.page_size - 1), 0);
-      float s = 0.f;
-      for (int d = 0; d < dk; ++d) s = fmaf(qs[d], to_float<T>(kr[d]), s);
-      m = fmaxf(m, s * scale);
+  if (weighting == 0) {
+    for (int base = 0; base < blocks; base += 64)
+      if (base + lane < blocks) m = fmaxf(m, score(pooled, base + lane));
+    for (int base = first & ~63; base <= pos; base += 64) {
+      const int j = base + lane;
+      if (j >= first && j <= pos) m = fmaxf(m, score(cache, j));
     }
   }
   m = wave_max(m);
@@ -177,37 +274,42 @@ __global__ __launch_bounds__(64) void attention_kv_plain_kernel(
   float o[kMaxDvPerLane];
 #pragma unroll
   for (int r = 0; r < kMaxDvPerLane; ++r) o[r] = 0.f;
-  for (int base = 0; base <= pos; base += 64) {
-    const int j = base + lane;
-    float e = 0.f;
-    if (j <= pos) {
-      const T* kr = cache + lay.key_offset(bt[j >> lay.page_shift], kvh, j & (lay.page_size - 1), 0);
-      float s = 0.f;
-      for (int d = 0; d < dk; ++d) s = fmaf(qs[d], to_float<T>(kr[d]), s);
-      e = weighting == 0 ? expf(s * scale - m) : 1.0f / (1.0f + expf(-(s * scale + sink)));
-      lsum += e;
-    }
-    __syncthreads();
-    es[lane] = e;
-    __syncthreads();
-    const int je = min(base + 63, pos);
-    for (int jj = base; jj <= je; ++jj) {
-      const float w = es[jj - base];
-      const int page = bt[jj >> lay.page_shift], slot = jj & (lay.page_size - 1);
+  // entries [from, to] of a section, 64 at a time from a multiple of 64: lane (j mod 64) owns entry j
+  auto walk = [&](const T* section, int from, int to) {
+    for (int base = from & ~63; base <= to; base += 64) {
+      const int j = base + lane;
+      float e = 0.f;
+      if (j >= from && j <= to) {
+        const float s = score(section, j);
+        e = weighting == 0 ? expf(s - m) : 1.0f / (1.0f + expf(-(s + sink)));
+        lsum += e;
+      }
+      __syncthreads();
+      es[lane] = e;
+      __syncthreads();
+      const int je = min(base + 63, to);
+      for (int jj = max(base, from); jj <= je; ++jj) {
+        const float w = es[jj - base];
+        const int page = bt[jj >> lay.page_shift], slot = jj & (lay.page_size - 1);
 #pragma unroll
-      for (int r = 0; r < kMaxDvPerLane; ++r) {
-        const int d = lane + 64 * r;
-        if (d < dv) o[r] = fmaf(w, to_float<T>(cache[lay.value_offset(page, kvh, slot, d)]), o[r]);
+        for (int r = 0; r < kMaxDvPerLane; ++r) {
+          const int d = lane + 64 * r;
+          if (d < dv) o[r] = fmaf(w, to_float<T>(section[lay.value_offset(page, kvh, slot, d)]), o[r]);
+        }
       }
     }
-  }
+  };
+  if (blocks > 0) walk(pooled, 0, blocks - 1);
+  walk(cache, first, pos);
   lsum = wave_sum(lsum);
   if (has_sink) lsum += expf(sink - m);
   if (weighting != 0) lsum = 1.0f;
+  // a gate a head: the head's result times sigmoid(gate[t][h])
+  const float g = gate != nullptr ? 1.0f / (1.0f + expf(-to_float<T>(gate[(int64_t)t * ld_gate + h]))) : 1.0f;
 #pragma unroll
   for (int r = 0; r < kMaxDvPerLane; ++r) {
     const int d = lane + 64 * r;
-    if (d < dv) out[(int64_t)t * ld_out + (int64_t)h * dv + d] = from_float<T>(o[r] / lsum);
+    if (d < dv) out[(int64_t)t * ld_out + (int64_t)h * dv + d] = from_float<T>(o[r] / lsum * g);
   }
 }
 
@@ -344,12 +446,70 @@ HFEE_API int hfee_qk_norm_write(void* q, int64_t ldq, int num_heads, const void*
   return 0;
 }
 
+HFEE_API int hfee_rotate_norm_write(void* q_out, int64_t ldqo, const float* q, int64_t ldq, int num_heads, const float* k,
+                                    int64_t ldk, const float* v, int64_t ldv, float value_eps, int dtype, const float* cos_t,
+                                    const float* sin_t, int half, int table_positions, int max_position,
+                                    const int* positions, const int* token_segment, const int* block_tables, int bt_stride,
+                                    void* cache, int kv_heads, int dk, int dv, int page_size, int sections, int n,
+                                    hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && num_heads > 0 && q != nullptr && q_out != nullptr, "rotate_norm_write: bad arguments");
+  if (n == 0) return 0;
+  HFEE_REQUIRE(half >= 0 && 2 * half <= dk && (half == 0 || (cos_t != nullptr && sin_t != nullptr)),
+               "rotate_norm_write: the rotated dims do not fit the heads, or their tables are missing");
+  HFEE_REQUIRE(half == 0 || max_position < table_positions,
+               "rotate_norm_write: position %d is beyond the rotation tables of %d positions", max_position, table_positions);
+  KvLayout lay;
+  if (make_kv_layout(&lay, kv_heads, dk, dv, page_size, sections)) return 1;
+  HFEE_REQUIRE(ldq >= (int64_t)num_heads * dk && ldqo >= (int64_t)num_heads * dk, "rotate_norm_write: q rows too short");
+  if (k != nullptr) {
+    HFEE_REQUIRE(v != nullptr && cache != nullptr && token_segment != nullptr && block_tables != nullptr,
+                 "rotate_norm_write: k, v, the cache and the block tables come together");
+    HFEE_REQUIRE(ldk >= (int64_t)kv_heads * dk && ldv >= (int64_t)kv_heads * dv, "rotate_norm_write: k/v rows too short");
+  }
+  const int64_t items = (int64_t)n * (num_heads + (k != nullptr ? 2 * kv_heads : 0));
+  HFEE_REQUIRE((items + 3) / 4 <= 0x7fffffff, "rotate_norm_write: too much work for one launch");
+#define LAUNCH(T)                                                                                                    \
+  rotate_norm_write_kernel<T><<<(unsigned)((items + 3) / 4), 256, 0, stream>>>((T*)q_out, ldqo, q, ldq, num_heads, k, ldk, v, \
+      ldv, value_eps, cos_t, sin_t, half, positions, token_segment, block_tables, bt_stride, (T*)cache, lay, n)
+  if (dtype == 0) LAUNCH(float);
+  else if (dtype == 1) LAUNCH(bf16_t);
+  else return fail("rotate_norm_write: unknown dtype %d", dtype);
+#undef LAUNCH
+  HFEE_CHECK_LAUNCH("rotate_norm_write");
+  return 0;
+}
+
+HFEE_API int hfee_kv_pool_write(void* cache, int dtype, int pool, const int* positions, const int* token_segment,
+                                const int* block_tables, int bt_stride, int kv_heads, int dk, int dv, int page_size, int n,
+                                hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && pool >= 1 && cache != nullptr, "kv_pool_write: bad arguments");
+  if (n == 0) return 0;
+  KvLayout lay;
+  if (make_kv_layout(&lay, kv_heads, dk, dv, page_size, 2)) return 1;
+  const int64_t items = (int64_t)n * kv_heads;
+  HFEE_REQUIRE((items + 3) / 4 <= 0x7fffffff, "kv_pool_write: too much work for one launch");
+  const int64_t pool_offset = (int64_t)page_size * (dk + dv);
+#define LAUNCH(T)                                                                                                    \
+  kv_pool_write_kernel<T><<<(unsigned)((items + 3) / 4), 256, 0, stream>>>((T*)cache, lay, pool, pool_offset, positions,  \
+      token_segment, block_tables, bt_stride, n)
+  if (dtype == 0) LAUNCH(float);
+  else if (dtype == 1) LAUNCH(bf16_t);
+  else return fail("kv_pool_write: unknown dtype %d", dtype);
+#undef LAUNCH
+  HFEE_CHECK_LAUNCH("kv_pool_write");
+  return 0;
+}
+
 HFEE_API int hfee_attention_kv_plain(void* out, int64_t ld_out, const void* q, int64_t ldq, const void* cache,
                                      int dtype, const int* positions, const int* token_segment,
                                      const int* block_tables, int bt_stride, int num_heads, int kv_heads, int dk,
-                                     int dv, int page_size, float scale, const float* sinks, int weighting, int n,
+                                     int dv, int page_size, float scale, const float* sinks, int weighting, int window,
+                                     int pool, float softcap, int sections, const void* gate, int64_t ld_gate, int n,
                                      hipStream_t stream) {
   HFEE_REQUIRE(n >= 0, "attention_kv_plain: bad token count");
+  KeySight sight;
+  if (make_key_sight(&sight, window, pool, softcap, sections, page_size, dk, dv)) return 1;
+  HFEE_REQUIRE(gate == nullptr || ld_gate >= num_heads, "attention_kv_plain: the gates' rows are too short");
   HFEE_REQUIRE(weighting == 0 || weighting == 1, "attention_kv_plain: the weights are a softmax's (0) or sigmoids (1)");
   if (n == 0) return 0;
   HFEE_REQUIRE(num_heads > 0 && kv_heads > 0 && num_heads % kv_heads == 0,
@@ -359,15 +519,17 @@ HFEE_API int hfee_attention_kv_plain(void* out, int64_t ld_out, const void* q, i
   HFEE_REQUIRE(num_heads <= 65535, "attention_kv_plain: too many heads");
   HFEE_REQUIRE(ldq >= (int64_t)num_heads * dk && ld_out >= (int64_t)num_heads * dv, "attention_kv_plain: q/out row too short");
   KvLayout lay;
-  if (make_kv_layout(&lay, kv_heads, dk, dv, page_size)) return 1;
+  if (make_kv_layout(&lay, kv_heads, dk, dv, page_size, sections)) return 1;
   dim3 grid(n, num_heads);
   const size_t lds = (dk + 64) * sizeof(float);
   if (dtype == 0)
     attention_kv_plain_kernel<float><<<grid, 64, lds, stream>>>((float*)out, ld_out, (const float*)q, ldq,
-        (const float*)cache, lay, positions, token_segment, block_tables, bt_stride, num_heads, scale, sinks, weighting);
+        (const float*)cache, lay, positions, token_segment, block_tables, bt_stride, num_heads, scale, sinks, weighting,
+        sight, (const float*)gate, ld_gate);
   else if (dtype == 1)
     attention_kv_plain_kernel<bf16_t><<<grid, 64, lds, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq,
-        (const bf16_t*)cache, lay, positions, token_segment, block_tables, bt_stride, num_heads, scale, sinks, weighting);
+        (const bf16_t*)cache, lay, positions, token_segment, block_tables, bt_stride, num_heads, scale, sinks, weighting,
+        sight, (const bf16_t*)gate, ld_gate);
   else
     return fail("attention_kv_plain: unknown dtype %d", dtype);
   HFEE_CHECK_LAUNCH("attention_kv_plain");

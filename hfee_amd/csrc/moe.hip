@@ -347,17 +347,32 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x,
 // with the same answer.  The sigmoid grows with its argument, so the largest scores are the largest logits.
 constexpr int kRouterMostExperts = 64 * 128;
 
+// score_kind 0: a score is sigmoid(z); 1: the softmax of z over all experts.  correction (float32 [experts] or
+// null) is added to a score where the experts are chosen and nowhere else: the weights are the scores.
 __global__ __launch_bounds__(256) void router_topk_kernel(const float* __restrict__ logits, int64_t ld, int n, int experts,
-                                                          int top, int* __restrict__ chosen, float* __restrict__ weights) {
+                                                          int top, int* __restrict__ chosen, float* __restrict__ weights,
+                                                          int score_kind, const float* __restrict__ correction) {
   const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (t >= n) return;
   const float* z = logits + (int64_t)t * ld;
+  float zmax = 0.f, inv_sum = 1.f;
+  if (score_kind == 1) {
+    zmax = -INFINITY;
+    for (int e = lane; e < experts; e += 64) zmax = fmaxf(zmax, z[e]);
+    zmax = wave_max(zmax);
+    float sum = 0.f;
+    for (int e = lane; e < experts; e += 64) sum += expf(z[e] - zmax);
+    inv_sum = 1.0f / wave_sum(sum);
+  }
+  auto score = [&](int e) { return score_kind == 1 ? expf(z[e] - zmax) * inv_sum : 1.0f / (1.0f + expf(-z[e])); };
+  // without a correction the order of the scores is the order of the logits (both scores grow with them)
+  auto choice = [&](int e) { return correction != nullptr ? score(e) + correction[e] : z[e]; };
   unsigned long long taken[2] = {0ull, 0ull};
   for (int j = 0; j < top; ++j) {
     float best = -INFINITY;
     int at = 0x7fffffff;
     for (int e = lane, i = 0; e < experts; e += 64, ++i) {
-      const float v = z[e];
+      const float v = choice(e);
       if (!((taken[i >> 6] >> (i & 63)) & 1ull) && (at == 0x7fffffff || v > best)) { best = v; at = e; }
     }
 #pragma unroll
@@ -369,7 +384,7 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const float* __restric
     if ((at & 63) == lane) taken[(at >> 6) >> 6] |= 1ull << ((at >> 6) & 63);
     if (lane == 0) {
       chosen[(int64_t)t * top + j] = at;
-      weights[(int64_t)t * top + j] = 1.0f / (1.0f + expf(-best));
+      weights[(int64_t)t * top + j] = score(at);
     }
   }
 }
@@ -377,11 +392,12 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const float* __restric
 }  // namespace
 
 HFEE_API int hfee_router_topk(const float* logits, int64_t ld, int n, int experts, int top, int* chosen, float* weights,
-                              hipStream_t stream) {
+                              int score_kind, const float* correction, hipStream_t stream) {
+  HFEE_REQUIRE(score_kind == 0 || score_kind == 1, "router_topk: the scores are sigmoids (0) or a softmax (1)");
   HFEE_REQUIRE(n >= 0 && experts >= 1 && experts <= kRouterMostExperts && top >= 1 && top <= experts && ld >= experts,
                "router_topk: a token uses 1 to %d experts (of at most %d), not %d", experts, kRouterMostExperts, top);
   if (n == 0) return 0;
-  router_topk_kernel<<<(n + 3) / 4, 256, 0, stream>>>(logits, ld, n, experts, top, chosen, weights);
+  router_topk_kernel<<<(n + 3) / 4, 256, 0, stream>>>(logits, ld, n, experts, top, chosen, weights, score_kind, correction);
   HFEE_CHECK_LAUNCH("router_topk");
   return 0;
 }

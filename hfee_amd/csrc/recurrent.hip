@@ -602,6 +602,56 @@ HFEE_API int hfee_unit_heads(float* x, int64_t ldx, int heads, int dim, float ep
   return 0;
 }
 
+namespace {
+
+// Rotation of projections on their way into a recurrence, in float32: out[t][h][d] (float32) from x[t][h][d]
+// (the engine's dtype), `heads` heads of `dim` side by side (queries and keys of a token as one row).  The
+// first 2 * half dims of a head are turned by the token's position (pairs (i, i + half), tables
+// [positions][half]); heads from `scaled_from` on are multiplied by `factor` behind the rotation.
+template <typename T>
+__global__ __launch_bounds__(256) void rotate_rows_kernel(
+    float* __restrict__ out, int64_t ldo, const T* __restrict__ x, int64_t ldx, const int* __restrict__ positions,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t, int half, int heads, int dim, int scaled_from,
+    float factor) {
+  const int t = blockIdx.x;
+  const float* c = cos_t + (int64_t)positions[t] * half;
+  const float* s = sin_t + (int64_t)positions[t] * half;
+  const T* xr = x + (int64_t)t * ldx;
+  float* orow = out + (int64_t)t * ldo;
+  for (int e = blockIdx.y * blockDim.x + threadIdx.x; e < heads * dim; e += gridDim.y * blockDim.x) {
+    const int h = e / dim, d = e - h * dim;
+    float v = to_float<T>(xr[e]);
+    if (d < half) v = v * c[d] - to_float<T>(xr[e + half]) * s[d];
+    else if (d < 2 * half) v = v * c[d - half] + to_float<T>(xr[e - half]) * s[d - half];
+    orow[e] = h >= scaled_from ? v * factor : v;
+  }
+}
+
+}  // namespace
+
+HFEE_API int hfee_rotate_rows(float* out, int64_t ldo, const void* x, int64_t ldx, int dtype, const int* positions,
+                              const float* cos_t, const float* sin_t, int half, int table_positions, int max_position,
+                              int heads, int dim, int scaled_from, float factor, int n, hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && heads > 0 && dim > 0 && half >= 0 && 2 * half <= dim, "rotate_rows: bad sizes");
+  HFEE_REQUIRE(ldo >= (int64_t)heads * dim && ldx >= (int64_t)heads * dim, "rotate_rows: rows too short");
+  HFEE_REQUIRE(half == 0 || (cos_t != nullptr && sin_t != nullptr && max_position < table_positions),
+               "rotate_rows: position %d is beyond the rotation tables of %d positions", max_position, table_positions);
+  if (n == 0) return 0;
+  int parts = (heads * dim + 255) / 256;
+  if (parts > 16) parts = 16;
+  dim3 grid(n, parts);
+  if (dtype == 0)
+    rotate_rows_kernel<float><<<grid, 256, 0, stream>>>(out, ldo, (const float*)x, ldx, positions, cos_t, sin_t, half, heads,
+                                                        dim, scaled_from, factor);
+  else if (dtype == 1)
+    rotate_rows_kernel<bf16_t><<<grid, 256, 0, stream>>>(out, ldo, (const bf16_t*)x, ldx, positions, cos_t, sin_t, half,
+                                                         heads, dim, scaled_from, factor);
+  else
+    return fail("rotate_rows: unknown dtype %d", dtype);
+  HFEE_CHECK_LAUNCH("rotate_rows");
+  return 0;
+}
+
 HFEE_API int hfee_scan_gate(float* out, int64_t ldo, const void* z, int64_t ldz, int dtype, const float* bias,
                             const float* per_head, int head_width, int mode, float number, int first_columns, int n,
                             int width, hipStream_t stream) {
@@ -636,7 +686,7 @@ HFEE_API int hfee_linear_scan(float* out, int64_t ldo, float* state, const float
   HFEE_REQUIRE(rule == 0 || ((rule == 1 || rule == 2) && beta != nullptr && ldb >= heads),
                "linear_scan: rule 0, or rule 1 or 2 with a number a head and token");
   HFEE_REQUIRE(ldq >= (int64_t)qk_heads * dim && ldk >= (int64_t)qk_heads * dim && ldv >= (int64_t)heads * vdim &&
-               ldd >= (decay_per_head ? (int64_t)heads : (int64_t)heads * dim) && ldo >= (int64_t)heads * vdim, "linear_scan: rows too short");
+               (ldd >= (decay_per_head ? (int64_t)heads : (int64_t)heads * dim) || (decay_per_head && ldd == 0)) && ldo >= (int64_t)heads * vdim, "linear_scan: rows too short");
   const int columns = kScanWaves * kScanColumns;
   dim3 grid((vdim + columns - 1) / columns, heads, segments);
   const int per = (dim + kScanParts - 1) / kScanParts;

@@ -48,7 +48,10 @@ _CORE_SIGNATURES = {
     "hfee_read_stream": [P, L, P, I, I, P],
     "hfee_mfma_loop": [P, I, I, P],
     "hfee_kv_write": [P, L, I, I, I, P, L, I, P, L, P, I, P, I, P, P, P, I, P, P, I, I, I, P, I, I, I, I, I, P],
-    "hfee_attention_kv_plain": [P, L, P, L, P, I, P, P, P, I, I, I, I, I, I, F, P, I, I, P],
+    "hfee_attention_kv_plain": [P, L, P, L, P, I, P, P, P, I, I, I, I, I, I, F, P, I, I, I, F, I, P, L, I, P],
+    "hfee_rotate_norm_write": [P, L, P, L, I, P, L, P, L, F, I, P, P, I, I, I, P, P, P, I, P, I, I, I, I, I, I, P],
+    "hfee_kv_pool_write": [P, I, I, P, P, P, I, I, I, I, I, I, P],
+    "hfee_rotate_rows": [P, L, P, L, I, P, P, P, I, I, I, I, I, I, F, I, P],
     "hfee_qk_norm_write": [P, L, I, P, L, P, L, I, P, P, F, F, I, P, P, P, I, P, I, I, I, I, I, P],
     "hfee_head_linear": [P, L, L, P, L, L, P, I, I, I, I, I, I, P],
     "hfee_norm_add": [P, P, I, P, I, P, I, F, F, P, I, P, F, I, I, P],
@@ -63,7 +66,7 @@ _CORE_SIGNATURES = {
     "hfee_linear_scan": [P, L, P, P, L, P, L, P, L, P, L, P, L, P, P, P, I, I, I, I, I, I, I, P],
     "hfee_rglru_scan": [P, L, I, P, P, L, P, P, L, P, P, L, P, P, P, P, I, I, I, I, P, L, P],
     "hfee_gate_group_norm": [P, L, I, P, L, P, L, P, I, P, L, P, I, I, F, I, P],
-    "hfee_router_topk": [P, L, I, I, I, P, P, P],
+    "hfee_router_topk": [P, L, I, I, I, P, P, I, P, P],
     "hfee_add_table_rows": [P, I, I, P, I, P, P],
     "hfee_scaled_add": [P, P, F, P, F, L, P],
     "hfee_gated_norm_add": [P, P, P, F, F, P, I, L, P, P, F, P, I, P, F, I, I, P],

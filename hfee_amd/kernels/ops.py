@@ -792,10 +792,10 @@ def _qkv_rows(out, x, weight, q):
 
 # ------------------------------- attention with keys and values of sizes of their own, and a sink
 
-def _kv_cache(cache_layer, kv_heads, dk, dv, page_size, what):
+def _kv_cache(cache_layer, kv_heads, dk, dv, page_size, what, sections: int = 1):
     _check(cache_layer.is_contiguous() and cache_layer.dim() == 3 and
-           tuple(cache_layer.shape[1:]) == (kv_heads, page_size * (dk + dv)),
-           f"{what}: the cache layer must be [pages, kv_heads, page_size * (key size + value size)]")
+           tuple(cache_layer.shape[1:]) == (kv_heads, sections * page_size * (dk + dv)),
+           f"{what}: the cache layer must be [pages, kv_heads, sections * page_size * (key size + value size)]")
 
 
 def kv_write(q, k, v, positions, token_segment, block_tables, cos, sin, cache_layer, num_heads: int, kv_heads: int,
@@ -849,18 +849,29 @@ def kv_write(q, k, v, positions, token_segment, block_tables, cos, sin, cache_la
 KEY_WEIGHTS = {"softmax": 0, "sigmoid": 1}
 
 
+def _sight(window: int, pool: int, softcap: float, sections: int, what: str):
+    _check(window >= 0 and pool >= 0 and softcap >= 0 and sections in (1, 2), f"{what}: bad window, pool, softcap or sections")
+    _check(not pool or sections == 2, f"{what}: pooled blocks live in a page's second section")
+
+
 def attention_kv_plain(out, q, cache_layer, positions, token_segment, block_tables, num_heads: int, kv_heads: int,
-                       dk: int, dv: int, page_size: int, scale: float, sinks=None, weights: str = "softmax"):
+                       dk: int, dv: int, page_size: int, scale: float, sinks=None, weights: str = "softmax",
+                       window: int = 0, pool: int = 0, softcap: float = 0.0, sections: int = 1, gate=None):
     """One wave per (token, head), any sizes, both dtypes: token t of head h reads the keys
     0..pos of its sequence; `sinks` (float32 [num_heads] or None) joins the softmax's denominator.
-    weights "sigmoid": no softmax, a key weighs sigmoid(score + sinks[head]) and nothing is normalized."""
+    weights "sigmoid": no softmax, a key weighs sigmoid(score + sinks[head]) and nothing is normalized.
+    window > 0: only the last `window` positions, the token's own included; pool > 0: also one key and
+    value (a page's second section, under the block's number) for every block of `pool` positions that lies
+    wholly before the window; softcap > 0: a score s counts as softcap * tanh(s / softcap).
+    gate ([n, num_heads] in the tensors' dtype): head h's result is multiplied by sigmoid(gate[t, h])."""
     _check(weights in KEY_WEIGHTS, f"attention_kv: the weights are {sorted(KEY_WEIGHTS)}, not {weights!r}")
-    _gpu(out, q, cache_layer, positions, token_segment, block_tables, sinks)
+    _gpu(out, q, cache_layer, positions, token_segment, block_tables, sinks, gate)
     n, w, ldq = _rows2d(q, "attention_kv q")
     no, wo, ldo = _rows2d(out, "attention_kv out")
     _check(no == n and w == num_heads * dk and wo == num_heads * dv, "attention_kv: q/out shape")
     _check(q.dtype == out.dtype == cache_layer.dtype, "attention_kv: dtype mismatch")
-    _kv_cache(cache_layer, kv_heads, dk, dv, page_size, "attention_kv")
+    _sight(window, pool, softcap, sections, "attention_kv")
+    _kv_cache(cache_layer, kv_heads, dk, dv, page_size, "attention_kv", sections)
     _i32(positions, "attention_kv positions", n)
     _i32(token_segment, "attention_kv token_segment", n)
     _check(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.stride(1) == 1,
@@ -868,9 +879,65 @@ def attention_kv_plain(out, q, cache_layer, positions, token_segment, block_tabl
     if sinks is not None:
         _check(sinks.dtype == torch.float32 and sinks.is_contiguous() and sinks.numel() == num_heads,
                "attention_kv: sinks must be float32 [num_heads]")
+    ldg = 0
+    if gate is not None:
+        ng, wg, ldg = _rows2d(gate, "attention_kv gate")
+        _check(ng == n and wg == num_heads and gate.dtype == q.dtype, "attention_kv: gate [n, num_heads] in q's dtype")
     lib.core().call("hfee_attention_kv_plain", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), _dt(q),
                     _ptr(positions), _ptr(token_segment), _ptr(block_tables), block_tables.stride(0),
-                    num_heads, kv_heads, dk, dv, page_size, float(scale), _ptr(sinks), KEY_WEIGHTS[weights], n, _stream())
+                    num_heads, kv_heads, dk, dv, page_size, float(scale), _ptr(sinks), KEY_WEIGHTS[weights],
+                    int(window), int(pool), float(softcap), int(sections), _ptr(gate), ldg, n, _stream())
+
+
+def rotate_norm_write(q_out, q, k, v, positions, token_segment, block_tables, cos, sin, cache_layer, num_heads: int,
+                      kv_heads: int, dk: int, dv: int, page_size: int, max_position: int, value_eps=None, sections: int = 1):
+    """From float32 projections (behind a short convolution): q ([n, num_heads * dk]) rotated into q_out (the
+    cache's dtype), k rotated and v into the token's slot of `cache_layer`, v divided by its root mean square
+    over each head where value_eps is a number.  The first 2 * half dims of a head are rotated, pairs
+    (i, i + half); cos/sin float32 [positions, half] or None.  k and v None: the queries only."""
+    _gpu(q_out, q, k, v, positions, token_segment, block_tables, cos, sin, cache_layer)
+    n, wq, ldq = _f32rows(q, "rotate_norm_write q")
+    no, wo, ldqo = _rows2d(q_out, "rotate_norm_write q_out")
+    _check(no == n and wq == wo == num_heads * dk, "rotate_norm_write: q shapes")
+    _i32(positions, "rotate_norm_write positions", n)
+    ldk = ldv = 0
+    if k is not None:
+        nk, wk, ldk = _f32rows(k, "rotate_norm_write k")
+        nv, wv, ldv = _f32rows(v, "rotate_norm_write v")
+        _check(nk == nv == n and wk == kv_heads * dk and wv == kv_heads * dv and q_out.dtype == cache_layer.dtype,
+               "rotate_norm_write: k/v shapes, or the cache's dtype")
+        _kv_cache(cache_layer, kv_heads, dk, dv, page_size, "rotate_norm_write", sections)
+        _i32(token_segment, "rotate_norm_write token_segment", n)
+        _check(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.stride(1) == 1,
+               "rotate_norm_write: block tables")
+    half = table_positions = 0
+    if cos is not None:
+        _check(cos.shape == sin.shape and cos.dim() == 2 and cos.is_contiguous() and sin.is_contiguous()
+               and cos.dtype == sin.dtype == torch.float32, "rotate_norm_write: cos/sin tables")
+        table_positions, half = cos.shape
+    has_k = k is not None
+    lib.core().call("hfee_rotate_norm_write", _ptr(q_out), ldqo, _ptr(q), ldq, num_heads, _ptr(k), ldk, _ptr(v), ldv,
+                    -1.0 if value_eps is None else float(value_eps), _dt(q_out), _ptr(cos), _ptr(sin), half, table_positions,
+                    int(max_position), _ptr(positions), _ptr(token_segment if has_k else None),
+                    _ptr(block_tables if has_k else None), block_tables.stride(0) if has_k else 0,
+                    _ptr(cache_layer if has_k else None), kv_heads, dk, dv, page_size, int(sections), n, _stream())
+
+
+def kv_pool_write(cache_layer, pool: int, positions, token_segment, block_tables, kv_heads: int, dk: int, dv: int,
+                  page_size: int):
+    """Behind the launch that wrote a step's keys and values: every token at the last position of a block of
+    `pool` positions leaves the means of the block's keys and values, as the cache holds them, in the pages'
+    second section under the block's number."""
+    _gpu(cache_layer, positions, token_segment, block_tables)
+    n = positions.numel()
+    _check(pool >= 1, "kv_pool_write: a block holds at least one position")
+    _kv_cache(cache_layer, kv_heads, dk, dv, page_size, "kv_pool_write", 2)
+    _i32(positions, "kv_pool_write positions", n)
+    _i32(token_segment, "kv_pool_write token_segment", n)
+    _check(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.stride(1) == 1,
+           "kv_pool_write: block tables")
+    lib.core().call("hfee_kv_pool_write", _ptr(cache_layer), _dt(cache_layer), int(pool), _ptr(positions), _ptr(token_segment),
+                    _ptr(block_tables), block_tables.stride(0), kv_heads, dk, dv, page_size, n, _stream())
 
 
 def qk_norm_write(q, k, v, positions, token_segment, block_tables, cache_layer, q_weight, k_weight, eps: float,
@@ -1270,6 +1337,26 @@ def unit_heads(x, heads: int, dim: int, eps: float, factor: float = 1.0):
     lib.core().call("hfee_unit_heads", _ptr(x), ldx, heads, dim, float(eps), float(factor), n, _stream())
 
 
+def rotate_rows(out, x, positions, cos, sin, heads: int, dim: int, max_position: int, scaled_from: int | None = None,
+                factor: float = 1.0):
+    """out (float32 [n, heads * dim]) = x (the engine's dtype) with the first 2 * half dims of every head turned by
+    the token's position (pairs (i, i + half); cos/sin float32 [positions, half], or None for no rotation), and the
+    heads from `scaled_from` on multiplied by `factor` behind it."""
+    _gpu(out, x, positions, cos, sin)
+    n, w, ldx = _rows2d(x, "rotate_rows x")
+    no, wo, ldo = _f32rows(out, "rotate_rows out")
+    _check(no == n and w == wo == heads * dim, "rotate_rows: shapes")
+    _i32(positions, "rotate_rows positions", n)
+    half = table_positions = 0
+    if cos is not None:
+        _check(cos.shape == sin.shape and cos.dim() == 2 and cos.is_contiguous() and sin.is_contiguous()
+               and cos.dtype == sin.dtype == torch.float32, "rotate_rows: cos/sin tables")
+        table_positions, half = cos.shape
+    lib.core().call("hfee_rotate_rows", _ptr(out), ldo, _ptr(x), ldx, _dt(x), _ptr(positions), _ptr(cos), _ptr(sin), half,
+                    table_positions, int(max_position), heads, dim, heads if scaled_from is None else int(scaled_from),
+                    float(factor), n, _stream())
+
+
 SCAN_GATES = {"step_decay": 0, "root_sigmoid": 1, "sigmoid": 2, "cast": 3, "softplus": 4}
 
 
@@ -1320,12 +1407,16 @@ def linear_scan(out, state, q, k, v, decay, beta, segment_rows, segment_lengths,
     S <- S + k (beta (v - S^T k))^T; "scaled_add": S <- diag(decay) S + k (beta v)^T; out = S^T q.
     q, k: float32 [n, qk_heads * dim] (head h reads q/k head h // (heads / qk_heads)); v, out:
     [n, heads * vdim]; decay: [n, heads * dim], or with decay_per_head [n, heads], one number for all
-    of a head's rows; beta [n, heads]."""
+    of a head's rows (or [heads]: the same decays for every token); beta [n, heads]."""
     _gpu(out, state, q, k, v, decay, beta, segment_rows, segment_lengths, segment_slots)
     n, wq, ldq = _f32rows(q, "linear_scan q")
     nk, wk, ldk = _f32rows(k, "linear_scan k")
     nv, wv, ldv = _f32rows(v, "linear_scan v")
-    nd, wd, ldd = _f32rows(decay, "linear_scan decay")
+    if decay.dim() == 1:        # one row for every token
+        _check(decay_per_head and decay.dtype == torch.float32 and decay.is_contiguous(), "linear_scan: constant decays are float32 [heads]")
+        nd, wd, ldd = n, decay.numel(), 0
+    else:
+        nd, wd, ldd = _f32rows(decay, "linear_scan decay")
     no, wo, ldo = _f32rows(out, "linear_scan out")
     rules = {"decay_add": 0, "delta": 1, "scaled_add": 2}
     _check(rule in rules, f"linear_scan: rule is one of {sorted(rules)}")
@@ -1457,14 +1548,24 @@ def moe_up(act, h, w_gate, w_up, top: int, chosen=None, table=None, token_ids=No
                     _ptr(token_ids), top, E, F, width, n, _ptr(in_weights), _stream())
 
 
-def router_topk(chosen, weights, logits, top: int):
-    """chosen (int32 [n, top]) = the experts with the `top` largest scores sigmoid(logits) of each row
-    (float32 [n, experts]; of equal scores the lower number), weights (float32 [n, top]) their scores."""
-    _gpu(chosen, weights, logits)
+ROUTER_SCORES = {"sigmoid": 0, "softmax": 1}
+
+
+def router_topk(chosen, weights, logits, top: int, score: str = "sigmoid", correction=None):
+    """chosen (int32 [n, top]) = the experts with the `top` largest choice scores of each row of logits
+    (float32 [n, experts]; of equal ones the lower number), weights (float32 [n, top]) their scores.  A score
+    is sigmoid(logit), or with score "softmax" the softmax over the row; the choice score is the score plus
+    correction (float32 [experts]) where one is given, and the weights never hold it."""
+    _gpu(chosen, weights, logits, correction)
     n, E, ld = _f32rows(logits, "router_topk logits")
+    _check(score in ROUTER_SCORES, f"router_topk: the scores are {sorted(ROUTER_SCORES)}")
     _check(chosen.dtype == torch.int32 and chosen.is_contiguous() and tuple(chosen.shape) == (n, top), "router_topk: chosen int32 [n, top]")
     _check(weights.dtype == torch.float32 and weights.is_contiguous() and tuple(weights.shape) == (n, top), "router_topk: weights float32 [n, top]")
-    lib.core().call("hfee_router_topk", _ptr(logits), ld, n, E, int(top), _ptr(chosen), _ptr(weights), _stream())
+    if correction is not None:
+        _check(correction.dtype == torch.float32 and correction.is_contiguous() and correction.numel() == E,
+               "router_topk: correction float32 [experts]")
+    lib.core().call("hfee_router_topk", _ptr(logits), ld, n, E, int(top), _ptr(chosen), _ptr(weights), ROUTER_SCORES[score],
+                    _ptr(correction), _stream())
 
 
 def moe_down(x, act, w_down, top: int, weight: float = 1.0, pair_weights=None, chosen=None, table=None, token_ids=None,

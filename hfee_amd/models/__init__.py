@@ -1,2 +1,2 @@
 """Architectures.  Importing this package registers every architecture it holds."""
-from . import llama, ronavik, sabezen, vofezen  # noqa: F401
+from . import llama, ronavik, sabezen, saposun, vofezen  # noqa: F401

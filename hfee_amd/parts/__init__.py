@@ -7,10 +7,10 @@ from .norm import LayerNorm, RMSNorm
 from .rotary import Rotary, rope_frequencies
 from .attention import Attention
 from .mlp import DenseMLP, GatedMLP
-from .kv_attention import KvAttention, LatentAttention, SigmoidAttention
+from .kv_attention import KvAttention, LatentAttention, SigmoidAttention, WindowAttention
 from .embedding import Embedding, Head
 from .mix_attention import MixedAttention
-from .recurrent import GatedDelta, GatedLinearAttention, RealGatedRecurrentUnit, StateSpace
+from .recurrent import GatedDelta, GatedLinearAttention, RealGatedRecurrentUnit, Retention, StateSpace
 from .paired import SideBySide
 from .moe import RoutedMoE, TableMoE
 from .block import ParallelBlock, PreNormBlock, SandwichBlock

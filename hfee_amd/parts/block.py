@@ -16,7 +16,9 @@ returns).
 
 "parallel" has one norm whose output both sub-layers read: with h = norm(x),
 x += mixer(h) + feed_forward(h).  Both add their last product straight into the float32 stream, the
-mixer first; a layer may have no feed-forward.
+mixer first; a layer may have no feed-forward.  With the parameter `residual_scale` = m the layer adds
+m * (mixer(h) + feed_forward(h)): the sub-layers then add into float32 rows of their own, which join the
+stream in one launch.
 """
 from __future__ import annotations
 
@@ -223,6 +225,7 @@ class ParallelBlock(Part):
 
     def __init__(self, spec: LayerSpec, dtype: torch.dtype):
         self.spec, self.dtype, self.hidden = spec, dtype, spec.hidden
+        self.residual_scale = float(spec.get("residual_scale", 1.0))
         self.norm = lookup("norm", spec.mixer_norm.kind)(spec.mixer_norm, spec.name_of("mixer_norm", "norm.weight"))
         self.mixer = lookup("mixer", spec.mixer.kind)(spec.mixer, spec.name_of("mixer", "mixer."), dtype)
         self.feed_forward = None
@@ -252,6 +255,12 @@ class ParallelBlock(Part):
     def forward(self, ctx, x, entry):
         h = ctx.rows("block.normed", self.hidden)
         self.norm.forward(ctx, h, x)
-        self.mixer.forward_add(ctx, x, h, entry.cache, entry.writes_cache)
+        into = x
+        if self.residual_scale != 1.0:
+            into = ctx.rows("block.sublayer_rows", self.hidden, torch.float32)
+            into.zero_()
+        self.mixer.forward_add(ctx, into, h, entry.cache, entry.writes_cache)
         if self.feed_forward is not None:
-            self.feed_forward.forward_add(ctx, x, h)
+            self.feed_forward.forward_add(ctx, into, h)
+        if into is not x:
+            ops.scaled_add(x, into, self.residual_scale)

@@ -1,4 +1,4 @@
-"""Three mixers over one family of attention kernels, whose keys and values have sizes of their own.
+"""Four mixers over one family of attention kernels, whose keys and values have sizes of their own.
 
 "kv_attention": grouped attention.  H query heads over G key/value heads (query head h reads
 key/value head h // (H/G)), key size Dk, value size Dv; q and k are rotated in the first
@@ -18,6 +18,22 @@ since q_plain . (W_uk,h c) = (W_uk,h^T q_plain) . c, the query of head h becomes
 size rank + rotated dims), the weighted sum is taken over the latents themselves (value size =
 rank), and W_uv,h is applied to the result.  Prompt portions and single tokens then run the same
 kernels, and a token's logits do not depend on how its prompt was cut.
+
+With `window` a query sees the last `window` positions only, itself included.  With `own_keys` False the
+layer has no W_dkv: it reads the latent and the rotated key part that another layer of the same latent
+size, rotated part and rotation keeps (the schedule names that layer's cache), with its own W_uk and W_uv.
+The rotation's pairs may be (i, i + half) or (2i, 2i + 1): the score is a sum over the rotated dims, so for
+the second kind the rows of W_uq's and W_dkv's rotated parts are put in the order evens, odds when they are
+bound, and the kernels turn pairs (i, i + half) of that order.
+
+"window_attention": grouped attention over a sliding window with pooled blocks.  q, k and v may pass a
+short causal convolution a channel (`conv` taps, no bias, no activation; the last taps - 1 projections of a
+request are state); q and k are rotated; with `value_norm_eps` a head's value is divided by its root mean
+square and cached so; score = q.k * scale, with `softcap` c then c * tanh(score / c); a query sees the last
+`window` positions and, with `pool` = P, one key and one value for every block of P positions that lies
+wholly before the window (the means of the block's cached keys and values, made when the block's last token
+is written, in the second section of the layer's pages under the block's number); tokens and blocks share
+one softmax; with `head_gate` a head's result is multiplied by sigmoid(W_g h)_h.
 
 "sigmoid_attention": grouped attention without a softmax and without a rotation.  q and k are divided
 by their root mean square over each head (eps `norm_eps`) and multiplied by a weight of the head's size
@@ -64,11 +80,14 @@ def plan_items(plan, rows: int) -> None:
         plan.host["attention_kv.single_max_position"] = max([p for _, _, p, _ in singles], default=0)
 
 
-def attend(ctx, out, q, cache, tables, num_heads, kv_heads, dk, dv, scale, sinks, matrix: bool, weights: str = "softmax") -> None:
-    """weights "sigmoid": no softmax, `sinks` holds the number a head that joins every score."""
+def attend(ctx, out, q, cache, tables, num_heads, kv_heads, dk, dv, scale, sinks, matrix: bool, weights: str = "softmax",
+           sight=None, gate=None) -> None:
+    """weights "sigmoid": no softmax, `sinks` holds the number a head that joins every score.  sight: None, or
+    dict(window, pool, softcap, sections) of a mixer whose queries do not see every earlier key as it is."""
+    sight = sight or {}
     if not matrix:
         ops.attention_kv_plain(out, q, cache, ctx.positions, ctx.token_segment, tables, num_heads, kv_heads, dk, dv,
-                               ctx.page_size, scale, sinks, weights=weights)
+                               ctx.page_size, scale, sinks, weights=weights, gate=gate, **sight)
         return
     portions = ctx.extra[f"attention_kv.portions.{ops.attention_kv_rows(dk, dv, num_heads // kv_heads, weights)}"]
     singles = ctx.extra["attention_kv.singles"]
@@ -303,36 +322,51 @@ class LatentAttention(_KvMixer):
         self.q_rank, self.kv_rank = spec.get("q_rank"), spec.get("kv_rank")
         self.scale = float(spec.get("scale", (self.plain + self.rotated) ** -0.5))
         self.eps = float(spec.get("norm_eps", 1e-6))
+        self.window = int(spec.get("window", 0))
+        self.own_keys = bool(spec.get("own_keys", True))
         self.position = lookup("position", spec.position.kind)(spec.position) if spec.position else None
-        if self.position is not None and (self.position.pairing != 0 or self.position.rotary_dim != self.rotated):
-            raise ValueError("latent_attention rotates the whole rotated part, pairs (i, i + half)")
+        if self.position is not None and self.position.rotary_dim != self.rotated:
+            raise ValueError("latent_attention rotates the whole rotated part")
+        self.pairing = self.position.pairing if self.position is not None else 0
         self.names = self._names(spec, dict(q_down="q_a_proj.weight", q_norm="q_a_norm.weight", q_up="q_b_proj.weight",
                                             kv_down="kv_a_proj.weight", kv_norm="kv_a_norm.weight", k_up="k_b_proj.weight",
                                             v_up="v_b_proj.weight", o="o_proj.weight"))
         # the absorbed form: one key/value head, keys [latent | rotated part], values the latent
         self.dk_abs, self.dv_abs = self.kv_rank + self.rotated, self.kv_rank
         self.kernel_sizes = (self.dk_abs, self.dv_abs, self.num_heads)
-        self.down_width = self.q_rank + self.kv_rank + self.rotated
+        self.down_width = self.q_rank + (self.kv_rank + self.rotated if self.own_keys else 0)
         self.matrix = (self._matrix(self.dk_abs, self.dv_abs, self.num_heads * self.dk_abs, self.num_heads * self.dv_abs)
-                       and self.down_width % 8 == 0 and self.q_rank % 8 == 0)
+                       and self.down_width % 8 == 0 and self.q_rank % 8 == 0 and not self.window)
+        self.sight = dict(window=self.window) if self.window else None
 
     def tensor_specs(self):
         n, H = self.names, self.num_heads
+        own = [TensorSpec(n["kv_down"], (self.kv_rank + self.rotated, self.hidden)),
+               TensorSpec(n["kv_norm"], (self.kv_rank,), role="vector", init=("one_plus_normal",))] if self.own_keys else []
         return [TensorSpec(n["q_down"], (self.q_rank, self.hidden)),
                 TensorSpec(n["q_norm"], (self.q_rank,), role="vector", init=("one_plus_normal",)),
-                TensorSpec(n["q_up"], (H * (self.plain + self.rotated), self.q_rank)),
-                TensorSpec(n["kv_down"], (self.kv_rank + self.rotated, self.hidden)),
-                TensorSpec(n["kv_norm"], (self.kv_rank,), role="vector", init=("one_plus_normal",)),
+                TensorSpec(n["q_up"], (H * (self.plain + self.rotated), self.q_rank)), *own,
                 TensorSpec(n["k_up"], (H * self.plain, self.kv_rank)),
                 TensorSpec(n["v_up"], (H * self.dv, self.kv_rank)),
                 TensorSpec(n["o"], (self.hidden, H * self.dv))]
 
     def bind(self, tensors):
         n, H = self.names, self.num_heads
-        self.w_down = torch.cat([tensors.pop(n["q_down"]), tensors.pop(n["kv_down"])], dim=0).contiguous()
+        # pairs (2i, 2i + 1): the rotated rows in the order evens, odds, whose pairs are (i, i + half)
+        turn = torch.arange(self.rotated)
+        if self.pairing == 1:
+            turn = torch.cat([turn[0::2], turn[1::2]])
+        w_down = [tensors.pop(n["q_down"])]
+        self.kv_norm = None
+        if self.own_keys:
+            kv_down = tensors.pop(n["kv_down"])
+            w_down += [kv_down[:self.kv_rank], kv_down[self.kv_rank:][turn.to(kv_down.device)]]
+            self.kv_norm = tensors.pop(n["kv_norm"]).to(torch.float32).contiguous()
+        self.w_down = torch.cat(w_down, dim=0).contiguous()
         self.q_norm = tensors.pop(n["q_norm"]).to(torch.float32).contiguous()
-        self.kv_norm = tensors.pop(n["kv_norm"]).to(torch.float32).contiguous()
-        self.w_q_up = tensors.pop(n["q_up"]).contiguous()
+        q_up = tensors.pop(n["q_up"])
+        per_head = torch.cat([torch.arange(self.plain), self.plain + turn]).to(q_up.device)
+        self.w_q_up = q_up.view(H, self.plain + self.rotated, self.q_rank)[:, per_head].reshape(q_up.shape).contiguous()
         # per head, as [inputs][outputs]: W_uk,h^T maps the plain query dims onto the latent, W_uv,h the
         # weighted latent onto the head's values
         self.w_k_absorb = tensors.pop(n["k_up"]).view(H, self.plain, self.kv_rank).contiguous()
@@ -345,10 +379,12 @@ class LatentAttention(_KvMixer):
 
     def key_layout(self):
         pos = self.position
-        return (1, self.dk_abs, self.dv_abs, None if pos is None else pos.signature())
+        return (1, self.dk_abs, self.dv_abs, None if pos is None else (pos.signature(), self.pairing))
 
     def forward_into(self, ctx, out, h, cache_layer: int, writes_cache: bool):
         n, H = ctx.n, self.num_heads
+        if writes_cache and not self.own_keys:
+            raise ValueError("a latent-attention layer without keys of its own reads another layer's cache")
         hn = h.tensor() if isinstance(h, LazyNorm) else h
         R, Dr, Dn = self.kv_rank, self.rotated, self.plain
         dk, dv = self.dk_abs, self.dv_abs
@@ -357,7 +393,7 @@ class LatentAttention(_KvMixer):
         pos = self.position
         cos, sin = (pos.cos, pos.sin) if pos else (None, None)
         down = ctx.rows("latent.down", self.down_width)
-        if writes_cache:
+        if writes_cache or not self.own_keys:
             product(ctx, down, hn, self.w_down, self.w_down_tiles)
         else:
             ops.linear(down[:, :self.q_rank], hn, self.w_down[:self.q_rank])
@@ -375,7 +411,118 @@ class LatentAttention(_KvMixer):
         ops.kv_write(qa, k, v, ctx.positions, ctx.token_segment, tables, cos, sin, cache, H, 1, dk, dk, dv, ctx.page_size,
                      ctx.max_position, q_rot_offset=R, k_rot_offset=R)
         att = ctx.rows("latent.mixed", H * dv)
-        attend(ctx, att, qa, cache, tables, H, 1, dk, dv, self.scale, None, self.matrix)
+        attend(ctx, att, qa, cache, tables, H, 1, dk, dv, self.scale, None, self.matrix, sight=self.sight)
         heads_out = ctx.rows("latent.values", H * self.dv)
         ops.head_linear(heads_out, att, self.w_v_expand, H, R, self.dv)
         product(ctx, out, heads_out, self.w_o, self.w_o_tiles)
+
+
+@register_mixer("window_attention")
+class WindowAttention(_KvMixer):
+    """Tensor names by role: q, k, v, o (matrices), q_conv, k_conv, v_conv ([channels, taps]), head_gate
+    ([heads, hidden])."""
+
+    def __init__(self, spec: MixerSpec, prefix: str, dtype: torch.dtype):
+        self.prefix, self.dtype = prefix, dtype
+        self.hidden = spec.get("hidden")
+        self.num_heads = spec.get("num_heads")
+        self.kv_heads = spec.get("num_kv_heads", self.num_heads)
+        self.dk = spec.get("key_dim")
+        self.dv = spec.get("value_dim", self.dk)
+        self.scale = float(spec.get("scale", self.dk ** -0.5))
+        self.softcap = float(spec.get("softcap", 0.0) or 0.0)
+        self.taps = int(spec.get("conv", 0) or 0)
+        self.window, self.pool = int(spec.get("window", 0) or 0), int(spec.get("pool", 0) or 0)
+        self.value_norm_eps = spec.get("value_norm_eps")          # None: the values as they are
+        self.has_gate = bool(spec.get("head_gate", False))
+        if self.num_heads % self.kv_heads:
+            raise ValueError(f"{self.num_heads} heads are not a multiple of {self.kv_heads} kv heads")
+        if self.window < 0 or self.pool < 0 or self.softcap < 0 or self.taps < 0:
+            raise ValueError("window, pool, softcap and conv are not negative")
+        if not self.window:
+            self.pool = 0                  # (without a window nothing ever lies before it)
+        self.position = lookup("position", spec.position.kind)(spec.position) if spec.position else None
+        if self.position is not None and self.position.pairing != 0:
+            raise ValueError("window_attention rotates pairs (i, i + half)")
+        self.names = self._names(spec, dict(q="q_proj.weight", k="k_proj.weight", v="v_proj.weight", o="o_proj.weight",
+                                            q_conv="q_conv.weight", k_conv="k_conv.weight", v_conv="v_conv.weight",
+                                            head_gate="gate_proj.weight"))
+        self.q_width, self.k_width, self.v_width = self.num_heads * self.dk, self.kv_heads * self.dk, self.kv_heads * self.dv
+        self.out_width = self.num_heads * self.dv
+        self.channels = self.q_width + self.k_width + self.v_width
+        self.sections = 2 if self.pool else 1
+        self.kernel_sizes = (self.dk, self.dv, self.num_heads // self.kv_heads)
+        self.matrix = False
+        self.sight = dict(window=self.window, pool=self.pool, softcap=self.softcap, sections=self.sections)
+
+    def tensor_specs(self):
+        n = self.names
+        specs = [TensorSpec(n["q"], (self.q_width, self.hidden)), TensorSpec(n["k"], (self.k_width, self.hidden)),
+                 TensorSpec(n["v"], (self.v_width, self.hidden)), TensorSpec(n["o"], (self.hidden, self.out_width))]
+        if self.taps:
+            specs += [TensorSpec(n["q_conv"], (self.q_width, self.taps), role="vector"),
+                      TensorSpec(n["k_conv"], (self.k_width, self.taps), role="vector"),
+                      TensorSpec(n["v_conv"], (self.v_width, self.taps), role="vector")]
+        if self.has_gate:
+            specs.append(TensorSpec(n["head_gate"], (self.num_heads, self.hidden)))
+        return specs
+
+    def bind(self, tensors):
+        n = self.names
+        # one product for everything that reads the layer's input: [q | k | v | a gate a head]
+        rows = [tensors.pop(n["q"]), tensors.pop(n["k"]), tensors.pop(n["v"])]
+        if self.has_gate:
+            rows.append(tensors.pop(n["head_gate"]))
+        self.w_in = torch.cat(rows, dim=0).contiguous()
+        self.w_o = tensors.pop(n["o"]).contiguous()
+        self.conv_taps = None
+        if self.taps:
+            self.conv_taps = torch.cat([tensors.pop(n[r]).to(torch.float32) for r in ("q_conv", "k_conv", "v_conv")], dim=0).contiguous()
+        self.w_in_tiles, self.w_o_tiles = tiles_of(self.dtype, self.w_in, self.w_o)
+
+    def cache_spec(self):
+        return CacheNeed("full", (self.kv_heads, self.sections, self.dk + self.dv), 0, layout=_LAYOUT)
+
+    def key_layout(self):
+        pos = self.position
+        return (self.kv_heads, self.dk, self.dv, self.sections, self.pool, self.taps, self.value_norm_eps,
+                None if pos is None else pos.signature())
+
+    def state_specs(self):
+        return [(self.prefix + "conv_state", (self.taps - 1, self.channels), self.dtype)] if self.taps else []
+
+    def prepare(self, info):
+        super().prepare(info)
+        self.conv_state = info.storage.states[self.prefix + "conv_state"] if self.taps else None
+
+    def forward_into(self, ctx, out, h, cache_layer: int, writes_cache: bool):
+        if not writes_cache:
+            raise ValueError("window_attention keeps its own keys: a request's convolution state belongs to one run of the layer")
+        hn = h.tensor() if isinstance(h, LazyNorm) else h
+        H, G, dk, dv = self.num_heads, self.kv_heads, self.dk, self.dv
+        cache = ctx.storage.layer(cache_layer, (G, self.sections * ctx.page_size * (dk + dv)))
+        tables = self._tables(ctx, cache_layer)
+        pos = self.position
+        cos, sin = (pos.cos, pos.sin) if pos else (None, None)
+        total = self.w_in.shape[0]       # (rows of a multiple of 8 elements, so that blocks of columns stay aligned)
+        proj = ctx.rows("window_attention.in", (total + 7) // 8 * 8)[:, :total]
+        product(ctx, proj, hn, self.w_in, self.w_in_tiles)
+        raw = proj[:, :self.channels]
+        qkv = ctx.rows("window_attention.qkv", self.channels, torch.float32)
+        if self.taps:
+            ops.short_conv_silu(qkv, raw, self.conv_state, self.conv_taps, ctx.token_segment, ctx.segment_rows,
+                                ctx.segment_slots, activation="none")
+            ops.short_conv_keep(self.conv_state, raw, ctx.segment_rows, ctx.segment_lengths, ctx.segment_slots)
+        else:
+            ops.scan_gate(qkv, raw, "cast")
+        q = ctx.rows("window_attention.q", self.q_width)
+        ops.rotate_norm_write(q, qkv[:, :self.q_width], qkv[:, self.q_width:self.q_width + self.k_width],
+                              qkv[:, self.q_width + self.k_width:], ctx.positions, ctx.token_segment, tables, cos, sin, cache,
+                              H, G, dk, dv, ctx.page_size, ctx.max_position, value_eps=self.value_norm_eps,
+                              sections=self.sections)
+        if self.pool:
+            ops.kv_pool_write(cache, self.pool, ctx.positions, ctx.token_segment, tables, G, dk, dv, ctx.page_size)
+        gate = proj[:, self.channels:self.channels + H] if self.has_gate else None
+        att = ctx.rows("kv_attention.out", self.out_width)
+        attend(ctx, att, q, cache, tables, H, G, dk, dv, self.scale, None, self.matrix, sight=self.sight, gate=gate)
+        product(ctx, out, att, self.w_o, self.w_o_tiles)

@@ -19,6 +19,12 @@ sigmoid(W_g2 W_g1 h); then the output product.
 S <- diag(a) S + k v^T; o = S^T q; each head's o normed as above with a weight shared by the heads,
 the heads side by side times silu(W_g h); then the output product.
 
+"retention": linear attention with a fixed decay a head and neither softmax nor denominator.  q, k
+(`num_heads` heads of `dim`) and v (heads of `vdim`) are plain products; q and k are rotated by the token's
+position (the position part's pairs (i, i + half)), k is then multiplied by dim^(-1/2);
+S <- decay_h S + k v^T, o = S^T q, with one decay a head from the spec; each head's o is divided by its root
+mean square (eps `norm_eps`, no weight), the heads side by side times silu(W_g h); then the output product.
+
 "state_space" (state-space duality): one product gives [z | x | B | C | dt] (z, x: `num_heads` heads of
 `vdim`; B, C: `groups` groups of `state`; dt a head).  x, B and C together pass a short causal convolution
 per channel with a bias and a SiLU.  dt = softplus(dt + dt_bias); per head (head h reads group
@@ -41,7 +47,7 @@ import torch.nn.functional as F
 from ..config.specs import MixerSpec
 from ..kernels import ops
 from ..weights.spec import TensorSpec
-from .base import LazyNorm, Mixer, register_mixer
+from .base import LazyNorm, Mixer, lookup, register_mixer
 from .kv_attention import product, tiles_of
 
 
@@ -209,6 +215,74 @@ class GatedLinearAttention(_StateMixer):
         ops.linear_scan(o, self.state, q, k, v, decay, None, rows, lengths, slots, H, H, D, V, "decay_add")
         gated = ctx.rows("gla.out", self.v_width)
         ops.head_norm_gate(gated, o, proj[:, self.at_g:self.at_a], self.norm_weight, H, V, self.norm_eps, "silu")
+        product(ctx, x, gated, self.w_o, self.w_o_tiles, add=True)
+
+
+@register_mixer("retention")
+class Retention(_StateMixer):
+    """Tensor names by role: q, k, v, g, o (matrices)."""
+
+    def __init__(self, spec: MixerSpec, prefix: str, dtype: torch.dtype):
+        self.prefix, self.dtype = prefix, dtype
+        self.hidden = spec.get("hidden")
+        self.heads = spec.get("num_heads")
+        self.dim, self.vdim = spec.get("dim"), spec.get("vdim")
+        self.decay = tuple(float(d) for d in spec.get("decay"))
+        self.norm_eps = float(spec.get("norm_eps", 1e-6))
+        if len(self.decay) != self.heads:
+            raise ValueError(f"{len(self.decay)} decays for {self.heads} heads")
+        self.position = lookup("position", spec.position.kind)(spec.position) if spec.position else None
+        if self.position is not None and self.position.pairing != 0:
+            raise ValueError("retention rotates pairs (i, i + half)")
+        self.names = self._names(spec, dict(q="q_proj.weight", k="k_proj.weight", v="v_proj.weight", g="g_proj.weight",
+                                            o="o_proj.weight"))
+        self.qk_width, self.v_width = self.heads * self.dim, self.heads * self.vdim
+
+    def tensor_specs(self):
+        n = self.names
+        return [TensorSpec(n["q"], (self.qk_width, self.hidden)), TensorSpec(n["k"], (self.qk_width, self.hidden)),
+                TensorSpec(n["v"], (self.v_width, self.hidden)), TensorSpec(n["g"], (self.v_width, self.hidden)),
+                TensorSpec(n["o"], (self.hidden, self.v_width))]
+
+    def bind(self, tensors):
+        n = self.names
+        # one product for everything that reads the layer's input: [q | k | v | g]
+        self.w_in = torch.cat([tensors.pop(n[r]) for r in ("q", "k", "v", "g")], dim=0).contiguous()
+        self.at_v = 2 * self.qk_width
+        self.at_g = self.at_v + self.v_width
+        self.w_o = tensors.pop(n["o"]).contiguous()
+        self.decays = torch.tensor(self.decay, dtype=torch.float32, device=self.w_o.device)
+        self.norm_weight = torch.ones(self.vdim, dtype=torch.float32, device=self.w_o.device)
+        self.w_in_tiles, self.w_o_tiles = tiles_of(self.dtype, self.w_in, self.w_o)
+
+    def state_specs(self):
+        return [(self.prefix + "state", (self.heads, *ops.scan_state_shape(self.dim, self.vdim)), torch.float32)]
+
+    def prepare(self, info):
+        self.state = info.storage.states[self.prefix + "state"]
+        if self.position is not None:
+            self.position.prepare(info.num_positions, info.device)
+
+    def forward_add(self, ctx, x, h, cache_layer: int, writes_cache: bool):
+        hn = h.tensor() if isinstance(h, LazyNorm) else h
+        H, D, V = self.heads, self.dim, self.vdim
+        rows, lengths, slots = self._segments(ctx)
+        total = self.w_in.shape[0]
+        proj = ctx.rows("retention.in", (total + 7) // 8 * 8)[:, :total]
+        product(ctx, proj, hn, self.w_in, self.w_in_tiles)
+        qkv = ctx.rows("retention.qkv", self.at_g, torch.float32)
+        pos = self.position
+        cos, sin = (pos.cos, pos.sin) if pos else (None, None)
+        # q and k as 2 H heads of one row: rotated, the keys' heads then times dim^(-1/2)
+        ops.rotate_rows(qkv[:, :self.at_v], proj[:, :self.at_v], ctx.positions, cos, sin, 2 * H, D, ctx.max_position,
+                        scaled_from=H, factor=D ** -0.5)
+        ops.scan_gate(qkv[:, self.at_v:], proj[:, self.at_v:self.at_g], "cast")
+        q, k, v = qkv[:, :self.qk_width], qkv[:, self.qk_width:self.at_v], qkv[:, self.at_v:]
+        o = ctx.rows("retention.read", self.v_width, torch.float32)
+        ops.linear_scan(o, self.state, q, k, v, self.decays, None, rows, lengths, slots, H, H, D, V, "decay_add",
+                        decay_per_head=True)
+        gated = ctx.rows("retention.out", self.v_width)
+        ops.head_norm_gate(gated, o, proj[:, self.at_g:], self.norm_weight, H, V, self.norm_eps, "silu")
         product(ctx, x, gated, self.w_o, self.w_o_tiles, add=True)
 
 
