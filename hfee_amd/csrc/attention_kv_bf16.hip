@@ -16,6 +16,15 @@
 //      split over several waves, whose partial results a second kernel joins.
 // The sink joins the denominator once, at the very end.
 //
+// A query may see less than every earlier key (`KeySight`, attention_kv.h): the last `window` positions only,
+// and beside them one pooled key and value for every block of `pool` positions that lies wholly before the
+// window (the second section of the pages, under the block's number); a score may be capped as
+// cap * tanh(score / cap); a head's result may be multiplied by sigmoid of a gate.  The kernel then walks
+// the tiles of the pooled section that any of its rows sees, and after them the token tiles from the one
+// that holds the first key of its first row's window; a key weighs where it lies within its row's bounds.
+// These run in the kernel that reads its operands straight from memory (not the one that shares key tiles
+// through LDS).
+//
 // Compiled with -DHFEE_KV_WEIGHTS=1 there is no softmax: a visible key weighs sigmoid(score + b_h), b_h a
 // number a head (given where the softmax has its sinks), nothing is normalized over the keys, and the
 // splits of a single token's keys are plain sums.
@@ -60,15 +69,30 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
 // quotient at the end does not depend on the reference), so most tiles cost no pass over the
 // output sums and no exchange between lanes.  Keys beyond the row's own position weigh nothing; `masked` says whether the tile
 // has any (the same answer in every lane).
+// A score as the weights take it, in base 2: s * scale, capped where a cap is given
+// (cap * tanh(x / cap), with tanh(y) = 1 - 2 / (e^(2y) + 1)).
+struct ScoreScale {
+  float scale_log2;      // scale * log2(e)
+  float twice_over_cap;  // 2 * scale * log2(e) / cap, or 0 without a cap
+  float cap_log2;        // cap * log2(e)
+  __device__ __forceinline__ float operator()(float s) const {
+    if (twice_over_cap == 0.f) return s * scale_log2;
+    const float e = __builtin_amdgcn_exp2f(s * twice_over_cap);
+    return cap_log2 * (1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f));
+  }
+};
+
+// `lo`, `hi`: the first and the last entry of the section that the lane's row sees.
 __device__ __forceinline__ void weigh_tile(f32x4 (&s)[2], float& reference, float& lsum, f32x4 (&acc)[VBLOCKS],
-                                           Operand& pop, int j0, int g, int pos, float scale_log2, bool masked) {
+                                           Operand& pop, int j0, int g, int lo, int hi, ScoreScale scaled, bool masked) {
   if constexpr (SIGMOID) {      // `reference` is the head's number (in base 2), and stays
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float p = 1.0f / (1.0f + __builtin_amdgcn_exp2f(-fmaf(s[kb][i], scale_log2, reference)));
-        s[kb][i] = masked && j0 + kb * 16 + g * 4 + i > pos ? 0.f : p;
+        const float p = 1.0f / (1.0f + __builtin_amdgcn_exp2f(-(scaled(s[kb][i]) + reference)));
+        const int j = j0 + kb * 16 + g * 4 + i;
+        s[kb][i] = masked && (j > hi || j < lo) ? 0.f : p;
       }
     pop.u = u32x4{pack_bf16(s[0][0], s[0][1]), pack_bf16(s[0][2], s[0][3]), pack_bf16(s[1][0], s[1][1]),
                   pack_bf16(s[1][2], s[1][3])};
@@ -79,8 +103,9 @@ __device__ __forceinline__ void weigh_tile(f32x4 (&s)[2], float& reference, floa
   for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      float v = s[kb][i] * scale_log2;
-      if (masked && j0 + kb * 16 + g * 4 + i > pos) v = -INFINITY;
+      float v = scaled(s[kb][i]);
+      const int j = j0 + kb * 16 + g * 4 + i;
+      if (masked && (j > hi || j < lo)) v = -INFINITY;
       s[kb][i] = v;
       tmax = fmaxf(tmax, v);
     }
@@ -137,8 +162,9 @@ template <int MODE, int RB>
 __global__ __launch_bounds__(256) void attention_kv_kernel(
     bf16_t* __restrict__ out, int64_t ld_out, const bf16_t* __restrict__ q, int64_t ldq,
     const bf16_t* __restrict__ cache, KvLayout lay, const int* __restrict__ items, int num_items,
-    const int* __restrict__ block_tables, int bt_stride, int num_heads, float scale_log2,
-    const float* __restrict__ sinks, float* __restrict__ partial, int splits) {
+    const int* __restrict__ block_tables, int bt_stride, int num_heads, ScoreScale scaled,
+    const float* __restrict__ sinks, float* __restrict__ partial, int splits, KeySight sight,
+    const bf16_t* __restrict__ gate, int64_t ld_gate) {
   const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
   const int hpg = num_heads / lay.kv_heads;
   const int groups16 = (hpg + 15) / 16;
@@ -191,22 +217,29 @@ __global__ __launch_bounds__(256) void attention_kv_kernel(
     for (int vb = 0; vb < VBLOCKS; ++vb) acc[b][vb] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  const int ntiles = (max_pos >> 5) + 1;
+  // the tiles to walk: those of the pooled section that any row sees, then the token tiles from the first
+  // key of the first row's window on (without a window or pooled blocks: the token tiles from the first)
+  const int pool_tiles = (sight.pooled_blocks(max_pos) + 31) >> 5;
+  const int tile_lo = sight.first_key(pos0) >> 5;
+  const int ntiles = pool_tiles + (max_pos >> 5) + 1 - tile_lo;
   const int per_split = (ntiles + splits - 1) / splits;
   const int tile_begin = split * per_split, tile_end = min(ntiles, tile_begin + per_split);
   const int last_block = max_pos >> lay.page_shift;
   const int slot_mask = lay.page_size - 1;
+  const bf16_t* const pooled = cache + sight.pool_offset;
 
   // the key operands of a tile: lane (r, g) holds dims 8g .. 8g+7 of every step of key r of each of the
   // tile's two blocks of 16 keys; `values` gets where the lane's value columns of the two blocks begin
-  auto load_keys = [&](int tile, Operand (&kop)[2][PIPE ? KSTEPS : 1], const bf16_t* (&values)[2]) {
+  auto load_keys = [&](int walked, Operand (&kop)[2][PIPE ? KSTEPS : 1], const bf16_t* (&values)[2]) {
+    const bf16_t* section = walked < pool_tiles ? pooled : cache;
+    const int tile = walked < pool_tiles ? walked : tile_lo + walked - pool_tiles;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
       const int jb = (tile << 5) + kb * 16;
       const int page = bt[min(jb >> lay.page_shift, last_block)];
       const int slot0 = jb & slot_mask;
-      const bf16_t* kr = cache + lay.key_offset(page, kvh, slot0 + r, g * 8);
-      values[kb] = cache + lay.values_of(page, kvh) + slot0 + g * 4;
+      const bf16_t* kr = section + lay.key_offset(page, kvh, slot0 + r, g * 8);
+      values[kb] = section + lay.values_of(page, kvh) + slot0 + g * 4;
 #pragma unroll
       for (int st = 0; st < (PIPE ? KSTEPS : 1); ++st) {
         if (st * 32 + g * 8 < DK) kop[kb][st].u = *reinterpret_cast<const u32x4*>(kr + st * 32);
@@ -215,13 +248,15 @@ __global__ __launch_bounds__(256) void attention_kv_kernel(
     }
   };
   // (without the second set, a key operand lives from its load to its products only)
-  auto load_keys_of_block = [&](int tile, int kb, int st, const bf16_t*& values) {
+  auto load_keys_of_block = [&](int walked, int kb, int st, const bf16_t*& values) {
+    const bf16_t* section = walked < pool_tiles ? pooled : cache;
+    const int tile = walked < pool_tiles ? walked : tile_lo + walked - pool_tiles;
     const int jb = (tile << 5) + kb * 16;
     const int page = bt[min(jb >> lay.page_shift, last_block)];
     const int slot0 = jb & slot_mask;
-    values = cache + lay.values_of(page, kvh) + slot0 + g * 4;
+    values = section + lay.values_of(page, kvh) + slot0 + g * 4;
     Operand one;
-    if (st * 32 + g * 8 < DK) one.u = *reinterpret_cast<const u32x4*>(cache + lay.key_offset(page, kvh, slot0 + r, g * 8) + st * 32);
+    if (st * 32 + g * 8 < DK) one.u = *reinterpret_cast<const u32x4*>(section + lay.key_offset(page, kvh, slot0 + r, g * 8) + st * 32);
     else one.u = u32x4{0, 0, 0, 0};
     return one;
   };
@@ -232,12 +267,21 @@ __global__ __launch_bounds__(256) void attention_kv_kernel(
   }
 
   for (int tile = tile_begin; tile < tile_end; ++tile) {
-    const int j0 = tile << 5;
-    // which row blocks see any key of this tile (the same answer in every lane)
-    bool live[RB];
+    const bool in_pool = tile < pool_tiles;
+    const int j0 = (in_pool ? tile : tile_lo + tile - pool_tiles) << 5;
+    // which row blocks see any key of this tile (the same answer in every lane), and whether all their rows
+    // see all of it: the entries that a row at position p sees are lo(p) .. hi(p), both growing with p
+    bool live[RB], masked_tile[RB];
 #pragma unroll
-    for (int b = 0; b < RB; ++b)
-      live[b] = MODE == 1 || (b < blocks && j0 <= pos0 + min(rows - 1, 16 * b + 15));
+    for (int b = 0; b < RB; ++b) {
+      const int p_first = MODE == 0 ? pos0 + min(rows - 1, 16 * b) : pos0;
+      const int p_last = MODE == 0 ? pos0 + min(rows - 1, 16 * b + 15) : pos0;
+      const int hi_first = in_pool ? sight.pooled_blocks(p_first) - 1 : p_first;
+      const int hi_last = in_pool ? sight.pooled_blocks(p_last) - 1 : p_last;
+      const int lo_first = in_pool ? 0 : sight.first_key(p_first), lo_last = in_pool ? 0 : sight.first_key(p_last);
+      live[b] = (MODE == 1 || b < blocks) && j0 <= hi_last && j0 + 31 >= lo_first;
+      masked_tile[b] = j0 + 31 > hi_first || j0 < lo_last;
+    }
     f32x4 s[RB][2];
     const bf16_t* vbase[2];
     if constexpr (PIPE) {
@@ -275,9 +319,9 @@ __global__ __launch_bounds__(256) void attention_kv_kernel(
 #pragma unroll
     for (int b = 0; b < RB; ++b) {
       if (!live[b]) continue;
-      // (the smallest position of the block's rows: a tile that ends at or before it hides no key)
-      const bool masked = j0 + 31 > (MODE == 0 ? pos0 + min(rows - 1, 16 * b) : pos0);
-      weigh_tile(s[b], m[b], lsum[b], acc[b], pop[b], j0, g, pos[b], scale_log2, masked);
+      const int lo = in_pool ? 0 : sight.first_key(pos[b]);
+      const int hi = in_pool ? sight.pooled_blocks(pos[b]) - 1 : pos[b];
+      weigh_tile(s[b], m[b], lsum[b], acc[b], pop[b], j0, g, lo, hi, scaled, masked_tile[b]);
     }
 #pragma unroll
     for (int vb = 0; vb < VBLOCKS; ++vb) {
@@ -313,7 +357,9 @@ __global__ __launch_bounds__(256) void attention_kv_kernel(
         l = l * a + exp2f(sk - m_all);
       }
       if (!valid[b]) continue;
-      const float inv = a / l;
+      float inv = a / l;
+      if (gate != nullptr)
+        inv *= 1.0f / (1.0f + __expf(-bf16_to_float(gate[(int64_t)token[b] * ld_gate + head[b]])));
       bf16_t* orow = out + (int64_t)token[b] * ld_out + (int64_t)head[b] * DV + g * 4;
 #pragma unroll
       for (int vb = 0; vb < VBLOCKS; ++vb) {
@@ -357,7 +403,7 @@ template <int RB>
 __global__ __launch_bounds__(256) void attention_kv_shared_kernel(
     bf16_t* __restrict__ out, int64_t ld_out, const bf16_t* __restrict__ q, int64_t ldq,
     const bf16_t* __restrict__ cache, KvLayout lay, const int* __restrict__ items, int num_items,
-    const int* __restrict__ block_tables, int bt_stride, int num_heads, float scale_log2,
+    const int* __restrict__ block_tables, int bt_stride, int num_heads, ScoreScale scaled,
     const float* __restrict__ sinks) {
   extern __shared__ __attribute__((aligned(16))) bf16_t stages[];
   const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4, w = threadIdx.x >> 6;
@@ -470,7 +516,7 @@ __global__ __launch_bounds__(256) void attention_kv_shared_kernel(
       if (!live[b]) continue;
       // (the smallest position of the block's rows: a tile that ends at or before it hides no key)
       const bool masked = j0 + 31 > pos0 + min(rows - 1, 16 * b);
-      weigh_tile(s[b], m[b], lsum[b], acc[b], pop[b], j0, g, pos[b], scale_log2, masked);
+      weigh_tile(s[b], m[b], lsum[b], acc[b], pop[b], j0, g, 0, pos[b], scaled, masked);
     }
 #pragma unroll
     for (int vb = 0; vb < VBLOCKS; ++vb) {
@@ -541,7 +587,7 @@ __global__ __launch_bounds__(256) void attention_kv_shared_kernel(
 // wave, and the value dims are then summed over the splits in their order, lanes over the dims.
 __global__ __launch_bounds__(64) void attention_kv_join_kernel(
     bf16_t* __restrict__ out, int64_t ld_out, const int* __restrict__ items, const float* __restrict__ partial,
-    int splits, int num_heads, const float* __restrict__ sinks) {
+    int splits, int num_heads, const float* __restrict__ sinks, const bf16_t* __restrict__ gate, int64_t ld_gate) {
   const int item = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const float* pr = partial + ((int64_t)item * num_heads + head) * splits * kPartial;
   const int token = items[item * 4];
@@ -552,7 +598,8 @@ __global__ __launch_bounds__(64) void attention_kv_join_kernel(
   // (0 for a split without keys and for lanes beyond the splits; without a softmax every split counts as it is)
   const float my_w = SIGMOID ? (lane < splits ? 1.f : 0.f) : exp2f(my_m - m);
   const float lsum = wave_sum(my_l * my_w) + (!SIGMOID && sinks != nullptr ? exp2f(sk - m) : 0.f);
-  const float inv = SIGMOID ? 1.0f : 1.0f / lsum;
+  float inv = SIGMOID ? 1.0f : 1.0f / lsum;
+  if (gate != nullptr) inv *= 1.0f / (1.0f + __expf(-bf16_to_float(gate[(int64_t)token * ld_gate + head])));
   for (int d = lane; d < DV; d += 64) {
     float o = 0.f;
 #pragma unroll 8
@@ -570,8 +617,9 @@ HFEE_API int hfee_attention_kv_bf16_dv() { return DV; }
 HFEE_API int hfee_attention_kv_bf16_weights() { return HFEE_KV_WEIGHTS; }
 // the most rows of an item of mode 0, for this many query heads a key/value head (where they are a
 // multiple of four, the kernel that shares the key tiles through LDS runs)
-HFEE_API int hfee_attention_kv_bf16_rows(int heads_per_kv_head) {
-  return 16 * (kSharedFits && heads_per_kv_head % 4 == 0 ? SHARED_BLOCKS : PORTION_BLOCKS);
+// (`plain_sight` 0: some keys are hidden, pooled, capped or gated, which the sharing kernel does not know)
+HFEE_API int hfee_attention_kv_bf16_rows(int heads_per_kv_head, int plain_sight) {
+  return 16 * (kSharedFits && heads_per_kv_head % 4 == 0 && plain_sight ? SHARED_BLOCKS : PORTION_BLOCKS);
 }
 
 // float32 words of `partial` that `splits` > 1 need for `num_items` single tokens
@@ -585,8 +633,13 @@ HFEE_API int hfee_attention_kv_bf16(void* out, int64_t ld_out, const void* q, in
                                     const int* items, int num_items, int mode, const int* block_tables,
                                     int bt_stride, int num_heads, int kv_heads, int page_size, float scale,
                                     const float* sinks, float* partial, int64_t partial_words, int splits,
-                                    hipStream_t stream) {
+                                    int window, int pool, float softcap, int sections, const void* gate,
+                                    int64_t ld_gate, hipStream_t stream) {
   HFEE_REQUIRE(num_items >= 0, "attention_kv_bf16: bad item count");
+  KeySight sight;
+  if (make_key_sight(&sight, window, pool, softcap, sections, page_size, DK, DV)) return 1;
+  HFEE_REQUIRE(gate == nullptr || ld_gate >= num_heads, "attention_kv_bf16: the gates' rows are too short");
+  const bool plain_sight = window == 0 && pool == 0 && softcap == 0.f && sections == 1 && gate == nullptr;
   if (num_items == 0) return 0;
   HFEE_REQUIRE(mode == 0 || mode == 1, "attention_kv_bf16: mode is 0 (portions) or 1 (single tokens)");
   HFEE_REQUIRE(num_heads > 0 && kv_heads > 0 && num_heads % kv_heads == 0,
@@ -600,14 +653,17 @@ HFEE_API int hfee_attention_kv_bf16(void* out, int64_t ld_out, const void* q, in
                partial_words >= hfee_attention_kv_bf16_partial(num_items, num_heads, splits)),
                "attention_kv_bf16: the partial results need more room");
   KvLayout lay;
-  if (make_kv_layout(&lay, kv_heads, DK, DV, page_size)) return 1;
+  if (make_kv_layout(&lay, kv_heads, DK, DV, page_size, sections)) return 1;
   const int hpg = num_heads / kv_heads;
   const int64_t units = mode == 0 ? num_heads : (int64_t)kv_heads * ((hpg + 15) / 16);
   const int64_t waves = (int64_t)num_items * splits * units;
   const int64_t blocks = (waves + 3) / 4;
   HFEE_REQUIRE(blocks <= 0x7fffffff, "attention_kv_bf16: too much work for one launch");
-  const float scale_log2 = scale * kLog2e;
-  if (mode == 0 && kSharedFits && hpg % 4 == 0) {
+  ScoreScale scaled;
+  scaled.scale_log2 = scale * kLog2e;
+  scaled.twice_over_cap = softcap > 0.f ? 2.0f * scale * kLog2e / softcap : 0.f;
+  scaled.cap_log2 = softcap * kLog2e;
+  if (mode == 0 && kSharedFits && hpg % 4 == 0 && plain_sight) {
     const size_t lds = 2 * (size_t)kStage * sizeof(bf16_t);
     static bool allowed = false;       // (more than 64 KB of LDS has to be asked for once)
     if (!allowed) {
@@ -620,17 +676,20 @@ HFEE_API int hfee_attention_kv_bf16(void* out, int64_t ld_out, const void* q, in
     HFEE_REQUIRE(groups <= 0x7fffffff, "attention_kv_bf16: too much work for one launch");
     attention_kv_shared_kernel<SHARED_BLOCKS><<<(unsigned)groups, 256, lds, stream>>>((bf16_t*)out, ld_out,
         (const bf16_t*)q, ldq, (const bf16_t*)cache, lay, items, num_items, block_tables, bt_stride, num_heads,
-        scale_log2, sinks);
+        scaled, sinks);
   } else if (mode == 0)
     attention_kv_kernel<0, PORTION_BLOCKS><<<(unsigned)blocks, 256, 0, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq,
-        (const bf16_t*)cache, lay, items, num_items, block_tables, bt_stride, num_heads, scale_log2, sinks, partial, 1);
+        (const bf16_t*)cache, lay, items, num_items, block_tables, bt_stride, num_heads, scaled, sinks, partial, 1, sight,
+        (const bf16_t*)gate, ld_gate);
   else
     attention_kv_kernel<1, 1><<<(unsigned)blocks, 256, 0, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq,
-        (const bf16_t*)cache, lay, items, num_items, block_tables, bt_stride, num_heads, scale_log2, sinks, partial, splits);
+        (const bf16_t*)cache, lay, items, num_items, block_tables, bt_stride, num_heads, scaled, sinks, partial, splits,
+        sight, (const bf16_t*)gate, ld_gate);
   HFEE_CHECK_LAUNCH("attention_kv_bf16");
   if (splits > 1) {
     attention_kv_join_kernel<<<dim3(num_items, num_heads), 64, 0, stream>>>((bf16_t*)out, ld_out, items, partial,
-                                                                            splits, num_heads, sinks);
+                                                                            splits, num_heads, sinks,
+                                                                            (const bf16_t*)gate, ld_gate);
     HFEE_CHECK_LAUNCH("attention_kv_bf16 join");
   }
   return 0;

@@ -976,10 +976,11 @@ def attention_kv_sizes_fit(dk: int, dv: int) -> bool:
     return dk % 16 == 0 and dv % 16 == 0 and 16 <= dk <= build.ATTENTION_KV_MOST[0] and 16 <= dv <= build.ATTENTION_KV_MOST[1]
 
 
-def attention_kv_rows(dk: int, dv: int, heads_per_kv_head: int = 1, weights: str = "softmax") -> int:
+def attention_kv_rows(dk: int, dv: int, heads_per_kv_head: int = 1, weights: str = "softmax", plain_sight: bool = True) -> int:
     """The most rows that an item of `attention_kv_bf16`'s mode 0 may hold for these sizes and this
-    many query heads a key/value head."""
-    return int(lib.attention_kv_bf16(dk, dv, weights).raw("hfee_attention_kv_bf16_rows")(int(heads_per_kv_head)))
+    many query heads a key/value head.  plain_sight False: for calls with a window, pooled blocks, a cap or a gate."""
+    return int(lib.attention_kv_bf16(dk, dv, weights).raw("hfee_attention_kv_bf16_rows")(int(heads_per_kv_head),
+                                                                                        1 if plain_sight else 0))
 
 
 def attention_kv_partial_words(num_items: int, num_heads: int, dv: int, splits: int) -> int:
@@ -988,17 +989,25 @@ def attention_kv_partial_words(num_items: int, num_heads: int, dv: int, splits: 
 
 def attention_kv_bf16(out, q, cache_layer, items, mode: int, block_tables, num_heads: int, kv_heads: int, dk: int,
                       dv: int, page_size: int, scale: float, sinks=None, partial=None, splits: int = 1,
-                      weights: str = "softmax"):
+                      weights: str = "softmax", window: int = 0, pool: int = 0, softcap: float = 0.0, sections: int = 1,
+                      gate=None):
     """Matrix-core attention, bfloat16 (weights: as in `attention_kv_plain`).  items: int32 [count, 4] on the device (first row, rows,
     first position, block-table row).  mode 0: an item is up to `attention_kv_rows` consecutive tokens of a portion;
     mode 1: an item is a single token (rows = 1), whose keys may be split over `splits` waves that
-    leave partial results in `partial` (float32, `attention_kv_partial_words`) for a joining kernel."""
-    _gpu(out, q, cache_layer, items, block_tables, sinks, partial)
+    leave partial results in `partial` (float32, `attention_kv_partial_words`) for a joining kernel.
+    window, pool, softcap, sections, gate: as in `attention_kv_plain`; with any of them an item of mode 0 holds
+    at most `attention_kv_rows(..., plain_sight=False)` rows."""
+    _gpu(out, q, cache_layer, items, block_tables, sinks, partial, gate)
+    _sight(window, pool, softcap, sections, "attention_kv")
     n, w, ldq = _rows2d(q, "attention_kv q")
     no, wo, ldo = _rows2d(out, "attention_kv out")
     _check(no == n and w == num_heads * dk and wo == num_heads * dv, "attention_kv: q/out shape")
     _check(q.dtype == out.dtype == cache_layer.dtype == torch.bfloat16, "attention_kv: bfloat16 tensors expected")
-    _kv_cache(cache_layer, kv_heads, dk, dv, page_size, "attention_kv")
+    _kv_cache(cache_layer, kv_heads, dk, dv, page_size, "attention_kv", sections)
+    ldg = 0
+    if gate is not None:
+        ng, wg, ldg = _rows2d(gate, "attention_kv gate")
+        _check(ng == n and wg == num_heads and gate.dtype == torch.bfloat16, "attention_kv: gate bfloat16 [n, num_heads]")
     _check(items.dtype == torch.int32 and items.dim() == 2 and items.shape[1] == 4 and items.is_contiguous(),
            "attention_kv: items must be [count, 4] int32")
     _check(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.stride(1) == 1,
@@ -1011,7 +1020,8 @@ def attention_kv_bf16(out, q, cache_layer, items, mode: int, block_tables, num_h
     lib.attention_kv_bf16(dk, dv, weights).call(
         "hfee_attention_kv_bf16", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), _ptr(items), items.shape[0], int(mode),
         _ptr(block_tables), block_tables.stride(0), num_heads, kv_heads, page_size, float(scale), _ptr(sinks),
-        _ptr(partial), 0 if partial is None else partial.numel(), int(splits), _stream())
+        _ptr(partial), 0 if partial is None else partial.numel(), int(splits), int(window), int(pool), float(softcap),
+        int(sections), _ptr(gate), ldg, _stream())
 
 
 def head_linear(out, x, weight, heads: int, n_in: int, n_out: int, tail: int = 0, x_head_stride: int | None = None,

@@ -89,16 +89,20 @@ def attend(ctx, out, q, cache, tables, num_heads, kv_heads, dk, dv, scale, sinks
         ops.attention_kv_plain(out, q, cache, ctx.positions, ctx.token_segment, tables, num_heads, kv_heads, dk, dv,
                                ctx.page_size, scale, sinks, weights=weights, gate=gate, **sight)
         return
-    portions = ctx.extra[f"attention_kv.portions.{ops.attention_kv_rows(dk, dv, num_heads // kv_heads, weights)}"]
+    plain_sight = not sight and gate is None
+    portions = ctx.extra[f"attention_kv.portions.{ops.attention_kv_rows(dk, dv, num_heads // kv_heads, weights, plain_sight)}"]
     singles = ctx.extra["attention_kv.singles"]
     if portions.shape[0]:
         ops.attention_kv_bf16(out, q, cache, portions, 0, tables, num_heads, kv_heads, dk, dv, ctx.page_size, scale, sinks,
-                              weights=weights)
+                              weights=weights, gate=gate, **sight)
     count = singles.shape[0]
     if count:
         # under a captured graph the split count is fixed for the whole width of the block table
         span = ctx.host.get("graph.max_context", ctx.host["attention_kv.single_max_position"] + 1)
         tiles = -(-span // _KEY_TILE)
+        if sight.get("window"):        # the window's tiles, and those of the pooled blocks before it
+            pooled = span // sight["pool"] if sight.get("pool") else 0
+            tiles = min(tiles, -(-sight["window"] // _KEY_TILE) + 1 + -(-pooled // _KEY_TILE))
         units = kv_heads * -(-(num_heads // kv_heads) // _ROWS)
         splits = max(1, min(tiles // 4, _WAVES_WANTED // (count * units), _MOST_SPLITS))
         partial = None
@@ -106,7 +110,7 @@ def attend(ctx, out, q, cache, tables, num_heads, kv_heads, dk, dv, scale, sinks
             partial = ctx.workspace.flat("attention_kv.partial", ops.attention_kv_partial_words(count, num_heads, dv, splits),
                                          torch.float32)
         ops.attention_kv_bf16(out, q, cache, singles, 1, tables, num_heads, kv_heads, dk, dv, ctx.page_size, scale, sinks,
-                              partial=partial, splits=splits, weights=weights)
+                              partial=partial, splits=splits, weights=weights, gate=gate, **sight)
 
 
 def tiles_of(dtype, *weights):
@@ -146,9 +150,11 @@ class _KvMixer(Mixer):
         if self.position is not None:
             self.position.prepare(info.num_positions, info.device)
 
+    plain_sight = True        # False in a mixer whose calls name a window, pooled blocks, a cap or a gate
+
     def plan(self, plan):
         if self.matrix:
-            plan_items(plan, ops.attention_kv_rows(*self.kernel_sizes, self.weights))
+            plan_items(plan, ops.attention_kv_rows(*self.kernel_sizes, self.weights, self.plain_sight))
 
     def forward_add(self, ctx, x, h, cache_layer: int, writes_cache: bool):
         y = ctx.rows("mixer.rows_out", self.hidden, torch.float32)
@@ -336,8 +342,9 @@ class LatentAttention(_KvMixer):
         self.kernel_sizes = (self.dk_abs, self.dv_abs, self.num_heads)
         self.down_width = self.q_rank + (self.kv_rank + self.rotated if self.own_keys else 0)
         self.matrix = (self._matrix(self.dk_abs, self.dv_abs, self.num_heads * self.dk_abs, self.num_heads * self.dv_abs)
-                       and self.down_width % 8 == 0 and self.q_rank % 8 == 0 and not self.window)
+                       and self.down_width % 8 == 0 and self.q_rank % 8 == 0)
         self.sight = dict(window=self.window) if self.window else None
+        self.plain_sight = not self.window
 
     def tensor_specs(self):
         n, H = self.names, self.num_heads
@@ -452,8 +459,9 @@ class WindowAttention(_KvMixer):
         self.channels = self.q_width + self.k_width + self.v_width
         self.sections = 2 if self.pool else 1
         self.kernel_sizes = (self.dk, self.dv, self.num_heads // self.kv_heads)
-        self.matrix = False
+        self.matrix = self._matrix(self.dk, self.dv, self.q_width, self.out_width)
         self.sight = dict(window=self.window, pool=self.pool, softcap=self.softcap, sections=self.sections)
+        self.plain_sight = False
 
     def tensor_specs(self):
         n = self.names

@@ -76,7 +76,7 @@ def latent_attention(h, w, pre, m, eps, shared=None):
     v = (c @ w[pre + "uv"].T).view(T, H, Dv)
     s = torch.einsum("ihd,jhd->hij", q_plain, k_plain) + torch.einsum("ihd,jd->hij", q_rot, kr)
     s = s * m["scale"]
-    s = s.masked_fill(~window_mask(T, m["mask"]["size"])[None], float("-inf"))
+    s = s.masked_fill(~window_mask(T, m["mask"]["size"] if m.get("mask") else T)[None], float("-inf"))
     p = torch.softmax(s, dim=-1)
     o = torch.einsum("hij,jhd->ihd", p, v).reshape(T, H * Dv)
     return o @ w[pre + "o"].T
@@ -124,8 +124,8 @@ def pooled_window_attention(h, w, pre, m, eps):
         q = rotate_half(q, pos, m["rot"]["dims"], m["rot"]["base"])
         k = rotate_half(k, pos, m["rot"]["dims"], m["rot"]["base"])
     v = rms(v, eps)
-    size = m["mask"]["size"]
-    P = m["mask"].get("pool", 0)
+    size = m["mask"]["size"] if m.get("mask") else T          # (without a mask: every earlier position)
+    P = m["mask"].get("pool", 0) if m.get("mask") else 0
     cap = m.get("softcap")
     out = torch.zeros(T, H, V, dtype=h.dtype)
     for i in range(T):
