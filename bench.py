@@ -77,6 +77,16 @@ RONAVIK_SIZES = {
     "4096-wide": dict(width=4096, heads=32, kv_heads=8, dim=128, expert_ff=2048),
 }
 
+# The Saposun design at the same two layer sizes, beside Sabezen (the closest of the other designs: parallel blocks,
+# attention, per-request states and experts): its layers go round latent attention over a window of 1,024 keys
+# (latents of 512 and 768 or 1,536, as Vofezen's), retention (heads of 128 key and 256 value channels, as many as
+# make the values as wide as the model), attention behind short convolutions over a window of 1,024 keys with pooled
+# blocks of 16 (heads and head size of the Llama layer of that width), and a latent layer that reads the first
+# one's keys; every layer has sixteen routed gated experts, two a token.
+SAPOSUN_SIZES = {
+    "2048-wide": dict(width=2048, heads=16, kv_heads=4, dim=128, expert_ff=1024, q_rank=768),
+    "4096-wide": dict(width=4096, heads=32, kv_heads=8, dim=128, expert_ff=2048, q_rank=1536),
+}
 
 CONTEXT = 8192
 PROMPT = 1024
@@ -135,6 +145,13 @@ def parse(argv=None):
                     help="with --ronavik: only this layer size")
     ap.add_argument("--ronavik-design", choices=["both", "ronavik", "sabezen"], default="both",
                     help="with --ronavik: only one of the two designs (for profiling)")
+    ap.add_argument("--saposun", action="store_true",
+                    help="the Saposun design beside Sabezen at equal layer sizes instead of the serving benchmark: its own "
+                    "JSON line, prefill of 2,048 tokens and decode at --batch")
+    ap.add_argument("--saposun-size", choices=sorted(SAPOSUN_SIZES), default=None,
+                    help="with --saposun: only this layer size")
+    ap.add_argument("--saposun-design", choices=["both", "saposun", "sabezen"], default="both",
+                    help="with --saposun: only one of the two designs (for profiling)")
     ap.add_argument("--no-extra-points", action="store_true",
                     help="skip the other shapes and the longer context that the default run adds under `points`")
     return ap.parse_args(argv)
@@ -254,6 +271,27 @@ def ronavik_config(size: dict, layers: int, vocab: int = 32000) -> dict:
             "layers": [dict((pair, ssm)[i % 2], mlp=moe) for i in range(layers)]}
 
 
+def saposun_config(size: dict, layers: int, vocab: int = 32000) -> dict:
+    d, H, G, hd = size["width"], size["heads"], size["kv_heads"], size["dim"]
+    latent = {"heads": H, "dim": hd, "rot_dim": 64, "vdim": hd, "q_rank": size["q_rank"], "kv_rank": 512,
+              "scale": (hd + 64) ** -0.5, "mask": {"size": 1024}, "rot": {"base": 500000.0, "dims": 64}}
+    lat = {"type": "latent_attention", "mixer": latent}
+    heads = d // 256
+    ret = {"type": "retention", "mixer": {"heads": heads, "dim": 128, "vdim": 256, "rot": {"base": 500000.0, "dims": 128},
+                                          "decay": [1.0 - 2.0 ** (-5 - 3 * i / max(1, heads - 1)) for i in range(heads)]}}
+    att = {"type": "attention", "mixer": {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "softcap": 30.0,
+                                          "conv": 4, "mask": {"size": 1024, "pool": 16}, "rot": {"base": 500000.0, "dims": hd}}}
+    moe = {"kind": "moe", "expert": {"ff": size["expert_ff"]}, "router": {"experts": 16, "top": 2}}
+    out = []
+    for i in range(layers):
+        layer = (lat, ret, att)[i % 3]
+        if i % 6 == 3:          # every other latent layer reads the keys of the one three layers before it
+            layer = {"type": "latent_attention", "mixer": dict(latent, kv_from=i - 3)}
+        out.append(dict(layer, mlp=moe))
+    return {"architecture": "Saposun", "vocab": vocab, "width": d, "norm": {"eps": 1e-5}, "residual_mult": 0.3,
+            "max_positions": 4096, "layers": out}
+
+
 def design_point(cj: dict, batch: int, steps: int, warmup: int) -> dict:
     """Prefill of 2,048 tokens and decode at `batch` requests of 1,024-token prompts for any
     registered architecture: times, and the fractions of the HBM and matrix peaks by the bytes a
@@ -286,13 +324,14 @@ def design_point(cj: dict, batch: int, steps: int, warmup: int) -> dict:
     chunked_flops = 0.0         # attention over chunks: the keys that a prompt of PREFILL tokens sees
     state_bytes = sum(4 * int(np.prod(shape)) for _, shape, dt in model.state_specs() if dt == torch.float32)
     scan_flops_a_token = 0      # the recurrences' multiply-adds on the vector units, counted apart
+    windows = []                # (elements a token, window, pool) of the cache layers that are read through a window
     mixers = [m for ls in spec.layers for m in ((ls.mixer.get("left"), ls.mixer.get("right"))
                                                 if ls.mixer.kind == "side_by_side" else (ls.mixer,))]
     for m in mixers:
         if m.kind == "mixed_attention":
             seen = sum(i % m.get("chunk") + 1 for i in range(PREFILL)) if m.get("chunk") else PREFILL * (PREFILL + 1) / 2
             chunked_flops += 2.0 * 2 * m.get("dim") * m.get("num_heads") * seen
-        elif m.kind in ("gated_delta", "gla"):
+        elif m.kind in ("gated_delta", "gla", "retention"):
             scan_flops_a_token += 2 * (4 if m.kind == "gated_delta" else 3) * m.get("num_heads") * m.get("dim") * m.get("vdim")
         elif m.kind == "state_space":
             scan_flops_a_token += 2 * 3 * m.get("num_heads") * m.get("state") * m.get("vdim")
@@ -302,8 +341,16 @@ def design_point(cj: dict, batch: int, steps: int, warmup: int) -> dict:
             attention_dims += 2 * m.get("head_dim") * m.get("num_heads")
         elif m.kind in ("kv_attention", "sigmoid_attention"):
             attention_dims += (m.get("key_dim") + m.get("value_dim")) * m.get("num_heads")
-        elif m.kind == "latent_attention":
-            attention_dims += (2 * m.get("kv_rank") + m.get("rotated_dim")) * m.get("num_heads")
+        elif m.kind in ("latent_attention", "window_attention"):
+            dims = ((2 * m.get("kv_rank") + m.get("rotated_dim")) if m.kind == "latent_attention"
+                    else m.get("key_dim") + m.get("value_dim")) * m.get("num_heads")
+            if m.get("window"):    # the keys of the window and the pooled blocks before it that a prompt of PREFILL tokens sees
+                w, p = m.get("window"), m.get("pool") or 0
+                seen = sum(min(i + 1, w) + ((i - w + 1) // p if p and i - w + 1 >= p else 0) for i in range(PREFILL))
+                chunked_flops += 2.0 * dims * seen
+                windows.append((dims // m.get("num_heads") * (m.get("num_kv_heads") or 1), w, p, m.get("own_keys", True)))
+            else:
+                attention_dims += dims
     page_size, context = 16, 4096
     engine = Engine(model, cache_tokens=batch * (PROMPT + steps + warmup + 4 * page_size) + PREFILL + page_size,
                     page_size=page_size, max_requests=max(batch, 2), max_batch_tokens=PREFILL, num_positions=context)
@@ -341,6 +388,9 @@ def design_point(cj: dict, batch: int, steps: int, warmup: int) -> dict:
     if chunks:
         context_read = context_read % min(chunks) + 1
     step_bytes = weight_bytes + batch * context_read * bytes_per_token(engine.groups, torch.bfloat16) + 2 * batch * state_bytes
+    for elements, w, p, own in windows:      # (a layer behind a window reads the window and the pooled blocks, not the context;
+        reads = min(context_read, w) + (context_read / p if p else 0)      # one that reads another layer's keys has no cache layer)
+        step_bytes -= batch * 2 * elements * ((context_read * (2 if p else 1) if own else 0) - reads)
     for r in list(sched.running):
         sched.cancel(r.request_id)
     while sched.has_work():
@@ -394,6 +444,24 @@ def ronavik_compare(args) -> dict:
             "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16", "layers": layers, "points": points}
 
 
+def saposun_compare(args) -> dict:
+    import hfee_amd  # noqa: F401
+    layers = args.layers or 6
+    points = {}
+    for name, size in SAPOSUN_SIZES.items():
+        if args.saposun_size not in (None, name):
+            continue
+        sab, _ = sabezen_configs(SABEZEN_SIZES[name], layers)
+        for design, cj in (("saposun", saposun_config(size, layers)), ("sabezen", sab)):
+            if args.saposun_design not in ("both", design):
+                continue
+            print(f"[bench] {design} {name}, {layers} layers", file=sys.stderr, flush=True)
+            points[f"{design}_{name}"] = design_point(cj, args.batch, min(args.steps, 32), min(args.warmup, 4))
+    return {"metric": "Saposun beside Sabezen at equal layer sizes: prefill of 2,048 tokens, decode at batch %d and "
+                      "1,024-token prompts (bf16, random weights)" % args.batch,
+            "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16", "layers": layers, "points": points}
+
+
 def sabezen_compare(args) -> dict:
     import hfee_amd  # noqa: F401
     layers = args.layers or 6
@@ -417,6 +485,9 @@ def main(argv=None) -> int:
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.saposun:
+        print(json.dumps(saposun_compare(args)), flush=True)
+        return 0
     if args.ronavik:
         print(json.dumps(ronavik_compare(args)), flush=True)
         return 0

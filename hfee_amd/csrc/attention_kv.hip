@@ -208,9 +208,17 @@ __global__ __launch_bounds__(256) void kv_pool_write_kernel(
   const float share = 1.0f / (float)pool;
   for (int d = lane; d < lay.dk + lay.dv; d += 64) {
     float sum = 0.f;
-    for (int j = pos - pool + 1; j <= pos; ++j) {
-      const int page = bt[j >> lay.page_shift], slot = j & (lay.page_size - 1);
-      sum += to_float<T>(cache[d < lay.dk ? lay.key_offset(page, g, slot, d) : lay.value_offset(page, g, slot, d - lay.dk)]);
+    for (int j0 = pos - pool + 1; j0 <= pos; j0 += 8) {       // eight loads on their way at a time, added in order
+      T part[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int j = min(j0 + i, pos);
+        const int page = bt[j >> lay.page_shift], slot = j & (lay.page_size - 1);
+        part[i] = cache[d < lay.dk ? lay.key_offset(page, g, slot, d) : lay.value_offset(page, g, slot, d - lay.dk)];
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (j0 + i <= pos) sum += to_float<T>(part[i]);
     }
     pooled[d < lay.dk ? lay.key_offset(to_page, g, to_slot, d) : lay.value_offset(to_page, g, to_slot, d - lay.dk)] =
         from_float<T>(sum * share);

@@ -22,8 +22,6 @@
 // cap * tanh(score / cap); a head's result may be multiplied by sigmoid of a gate.  The kernel then walks
 // the tiles of the pooled section that any of its rows sees, and after them the token tiles from the one
 // that holds the first key of its first row's window; a key weighs where it lies within its row's bounds.
-// These run in the kernel that reads its operands straight from memory (not the one that shares key tiles
-// through LDS).
 //
 // Compiled with -DHFEE_KV_WEIGHTS=1 there is no softmax: a visible key weighs sigmoid(score + b_h), b_h a
 // number a head (given where the softmax has its sinks), nothing is normalized over the keys, and the
@@ -404,7 +402,7 @@ __global__ __launch_bounds__(256) void attention_kv_shared_kernel(
     bf16_t* __restrict__ out, int64_t ld_out, const bf16_t* __restrict__ q, int64_t ldq,
     const bf16_t* __restrict__ cache, KvLayout lay, const int* __restrict__ items, int num_items,
     const int* __restrict__ block_tables, int bt_stride, int num_heads, ScoreScale scaled,
-    const float* __restrict__ sinks) {
+    const float* __restrict__ sinks, KeySight sight, const bf16_t* __restrict__ gate, int64_t ld_gate) {
   extern __shared__ __attribute__((aligned(16))) bf16_t stages[];
   const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4, w = threadIdx.x >> 6;
   const int hpg = num_heads / lay.kv_heads;
@@ -442,23 +440,30 @@ __global__ __launch_bounds__(256) void attention_kv_shared_kernel(
     for (int vb = 0; vb < VBLOCKS; ++vb) acc[b][vb] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
   const int max_pos = pos0 + rows - 1;
-  const int ntiles = (max_pos >> 5) + 1;
+  // the tiles to walk: those of the pooled section that any row sees, then the token tiles from the first key
+  // of the first row's window on
+  const int pool_tiles = (sight.pooled_blocks(max_pos) + 31) >> 5;
+  const int tile_lo = sight.first_key(pos0) >> 5;
+  const int ntiles = pool_tiles + (max_pos >> 5) + 1 - tile_lo;
   const int last_block = max_pos >> lay.page_shift;
   const int slot_mask = lay.page_size - 1;
+  const bf16_t* const pooled = cache + sight.pool_offset;
 
   // two sets of registers for the chunks on their way, where that is few registers: a tile is then
   // asked for two tiles before it is multiplied (memory takes longer than one tile's products)
   constexpr bool DEEP = 4 * (kKeyLoads + kValueLoads) <= 32;
   u32x4 kst_a[kKeyLoads], vst_a[kValueLoads], kst_b[DEEP ? kKeyLoads : 1], vst_b[DEEP ? kValueLoads : 1];
-  auto fetch = [&](int tile, u32x4* kst, u32x4* vst) {          // this thread's chunks of the tile, into registers
+  auto fetch = [&](int walked, u32x4* kst, u32x4* vst) {          // this thread's chunks of the tile, into registers
+    const bf16_t* section = walked < pool_tiles ? pooled : cache;
+    const int tile = walked < pool_tiles ? walked : tile_lo + walked - pool_tiles;
     const bf16_t* keys[2];
     const bf16_t* values[2];
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
       const int jb = (tile << 5) + kb * 16;
       const int page = bt[min(jb >> lay.page_shift, last_block)];
-      keys[kb] = cache + lay.key_offset(page, kvh, jb & slot_mask, 0);
-      values[kb] = cache + lay.values_of(page, kvh) + (jb & slot_mask);
+      keys[kb] = section + lay.key_offset(page, kvh, jb & slot_mask, 0);
+      values[kb] = section + lay.values_of(page, kvh) + (jb & slot_mask);
     }
 #pragma unroll
     for (int i = 0; i < kKeyLoads; ++i) {
@@ -490,11 +495,20 @@ __global__ __launch_bounds__(256) void attention_kv_shared_kernel(
       if (c < kValueChunks) *reinterpret_cast<u32x4*>(st + 32 * kKeyRow + (c >> 2) * kValueColumn + (c & 3) * 8) = vst[i];
     }
   };
-  auto multiply = [&](int tile, const bf16_t* st) {
-    const int j0 = tile << 5;
-    bool live[RB];
+  auto multiply = [&](int walked, const bf16_t* st) {
+    const bool in_pool = walked < pool_tiles;
+    const int j0 = (in_pool ? walked : tile_lo + walked - pool_tiles) << 5;
+    // (the entries that a row at position p sees are lo(p) .. hi(p), both growing with p)
+    bool live[RB], masked_tile[RB];
 #pragma unroll
-    for (int b = 0; b < RB; ++b) live[b] = b < blocks && j0 <= pos0 + min(rows - 1, 16 * b + 15);
+    for (int b = 0; b < RB; ++b) {
+      const int p_first = pos0 + min(rows - 1, 16 * b), p_last = pos0 + min(rows - 1, 16 * b + 15);
+      const int hi_first = in_pool ? sight.pooled_blocks(p_first) - 1 : p_first;
+      const int hi_last = in_pool ? sight.pooled_blocks(p_last) - 1 : p_last;
+      const int lo_first = in_pool ? 0 : sight.first_key(p_first), lo_last = in_pool ? 0 : sight.first_key(p_last);
+      live[b] = b < blocks && j0 <= hi_last && j0 + 31 >= lo_first;
+      masked_tile[b] = j0 + 31 > hi_first || j0 < lo_last;
+    }
     f32x4 s[RB][2];
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
@@ -514,9 +528,9 @@ __global__ __launch_bounds__(256) void attention_kv_shared_kernel(
 #pragma unroll
     for (int b = 0; b < RB; ++b) {
       if (!live[b]) continue;
-      // (the smallest position of the block's rows: a tile that ends at or before it hides no key)
-      const bool masked = j0 + 31 > pos0 + min(rows - 1, 16 * b);
-      weigh_tile(s[b], m[b], lsum[b], acc[b], pop[b], j0, g, 0, pos[b], scaled, masked);
+      const int lo = in_pool ? 0 : sight.first_key(pos[b]);
+      const int hi = in_pool ? sight.pooled_blocks(pos[b]) - 1 : pos[b];
+      weigh_tile(s[b], m[b], lsum[b], acc[b], pop[b], j0, g, lo, hi, scaled, masked_tile[b]);
     }
 #pragma unroll
     for (int vb = 0; vb < VBLOCKS; ++vb) {
@@ -571,7 +585,8 @@ __global__ __launch_bounds__(256) void attention_kv_shared_kernel(
       l = l * a + exp2f(sk - m_all);
     }
     if (!valid[b]) continue;
-    const float inv = a / l;
+    float inv = a / l;
+    if (gate != nullptr) inv *= 1.0f / (1.0f + __expf(-bf16_to_float(gate[(int64_t)token[b] * ld_gate + head])));
     bf16_t* orow = out + (int64_t)token[b] * ld_out + (int64_t)head * DV + g * 4;
 #pragma unroll
     for (int vb = 0; vb < VBLOCKS; ++vb) {
@@ -617,9 +632,8 @@ HFEE_API int hfee_attention_kv_bf16_dv() { return DV; }
 HFEE_API int hfee_attention_kv_bf16_weights() { return HFEE_KV_WEIGHTS; }
 // the most rows of an item of mode 0, for this many query heads a key/value head (where they are a
 // multiple of four, the kernel that shares the key tiles through LDS runs)
-// (`plain_sight` 0: some keys are hidden, pooled, capped or gated, which the sharing kernel does not know)
-HFEE_API int hfee_attention_kv_bf16_rows(int heads_per_kv_head, int plain_sight) {
-  return 16 * (kSharedFits && heads_per_kv_head % 4 == 0 && plain_sight ? SHARED_BLOCKS : PORTION_BLOCKS);
+HFEE_API int hfee_attention_kv_bf16_rows(int heads_per_kv_head) {
+  return 16 * (kSharedFits && heads_per_kv_head % 4 == 0 ? SHARED_BLOCKS : PORTION_BLOCKS);
 }
 
 // float32 words of `partial` that `splits` > 1 need for `num_items` single tokens
@@ -639,7 +653,6 @@ HFEE_API int hfee_attention_kv_bf16(void* out, int64_t ld_out, const void* q, in
   KeySight sight;
   if (make_key_sight(&sight, window, pool, softcap, sections, page_size, DK, DV)) return 1;
   HFEE_REQUIRE(gate == nullptr || ld_gate >= num_heads, "attention_kv_bf16: the gates' rows are too short");
-  const bool plain_sight = window == 0 && pool == 0 && softcap == 0.f && sections == 1 && gate == nullptr;
   if (num_items == 0) return 0;
   HFEE_REQUIRE(mode == 0 || mode == 1, "attention_kv_bf16: mode is 0 (portions) or 1 (single tokens)");
   HFEE_REQUIRE(num_heads > 0 && kv_heads > 0 && num_heads % kv_heads == 0,
@@ -663,7 +676,7 @@ HFEE_API int hfee_attention_kv_bf16(void* out, int64_t ld_out, const void* q, in
   scaled.scale_log2 = scale * kLog2e;
   scaled.twice_over_cap = softcap > 0.f ? 2.0f * scale * kLog2e / softcap : 0.f;
   scaled.cap_log2 = softcap * kLog2e;
-  if (mode == 0 && kSharedFits && hpg % 4 == 0 && plain_sight) {
+  if (mode == 0 && kSharedFits && hpg % 4 == 0) {
     const size_t lds = 2 * (size_t)kStage * sizeof(bf16_t);
     static bool allowed = false;       // (more than 64 KB of LDS has to be asked for once)
     if (!allowed) {
@@ -676,7 +689,7 @@ HFEE_API int hfee_attention_kv_bf16(void* out, int64_t ld_out, const void* q, in
     HFEE_REQUIRE(groups <= 0x7fffffff, "attention_kv_bf16: too much work for one launch");
     attention_kv_shared_kernel<SHARED_BLOCKS><<<(unsigned)groups, 256, lds, stream>>>((bf16_t*)out, ld_out,
         (const bf16_t*)q, ldq, (const bf16_t*)cache, lay, items, num_items, block_tables, bt_stride, num_heads,
-        scaled, sinks);
+        scaled, sinks, sight, (const bf16_t*)gate, ld_gate);
   } else if (mode == 0)
     attention_kv_kernel<0, PORTION_BLOCKS><<<(unsigned)blocks, 256, 0, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq,
         (const bf16_t*)cache, lay, items, num_items, block_tables, bt_stride, num_heads, scaled, sinks, partial, 1, sight,

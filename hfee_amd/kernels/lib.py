@@ -81,7 +81,7 @@ _ATTENTION_KV_SIGNATURES = {
     "hfee_attention_kv_bf16_dk": [],
     "hfee_attention_kv_bf16_dv": [],
     "hfee_attention_kv_bf16_weights": [],
-    "hfee_attention_kv_bf16_rows": [I, I],
+    "hfee_attention_kv_bf16_rows": [I],
     "hfee_attention_kv_bf16": [P, L, P, L, P, P, I, I, P, I, I, I, I, F, P, P, L, I, I, I, F, I, P, L, P],
 }
 

@@ -976,11 +976,10 @@ def attention_kv_sizes_fit(dk: int, dv: int) -> bool:
     return dk % 16 == 0 and dv % 16 == 0 and 16 <= dk <= build.ATTENTION_KV_MOST[0] and 16 <= dv <= build.ATTENTION_KV_MOST[1]
 
 
-def attention_kv_rows(dk: int, dv: int, heads_per_kv_head: int = 1, weights: str = "softmax", plain_sight: bool = True) -> int:
+def attention_kv_rows(dk: int, dv: int, heads_per_kv_head: int = 1, weights: str = "softmax") -> int:
     """The most rows that an item of `attention_kv_bf16`'s mode 0 may hold for these sizes and this
-    many query heads a key/value head.  plain_sight False: for calls with a window, pooled blocks, a cap or a gate."""
-    return int(lib.attention_kv_bf16(dk, dv, weights).raw("hfee_attention_kv_bf16_rows")(int(heads_per_kv_head),
-                                                                                        1 if plain_sight else 0))
+    many query heads a key/value head."""
+    return int(lib.attention_kv_bf16(dk, dv, weights).raw("hfee_attention_kv_bf16_rows")(int(heads_per_kv_head)))
 
 
 def attention_kv_partial_words(num_items: int, num_heads: int, dv: int, splits: int) -> int:
@@ -995,8 +994,7 @@ def attention_kv_bf16(out, q, cache_layer, items, mode: int, block_tables, num_h
     first position, block-table row).  mode 0: an item is up to `attention_kv_rows` consecutive tokens of a portion;
     mode 1: an item is a single token (rows = 1), whose keys may be split over `splits` waves that
     leave partial results in `partial` (float32, `attention_kv_partial_words`) for a joining kernel.
-    window, pool, softcap, sections, gate: as in `attention_kv_plain`; with any of them an item of mode 0 holds
-    at most `attention_kv_rows(..., plain_sight=False)` rows."""
+    window, pool, softcap, sections, gate: as in `attention_kv_plain`."""
     _gpu(out, q, cache_layer, items, block_tables, sinks, partial, gate)
     _sight(window, pool, softcap, sections, "attention_kv")
     n, w, ldq = _rows2d(q, "attention_kv q")

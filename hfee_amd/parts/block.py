@@ -258,8 +258,12 @@ class ParallelBlock(Part):
         into = x
         if self.residual_scale != 1.0:
             into = ctx.rows("block.sublayer_rows", self.hidden, torch.float32)
-            into.zero_()
-        self.mixer.forward_add(ctx, into, h, entry.cache, entry.writes_cache)
+        if into is not x and hasattr(self.mixer, "forward_into"):       # (the mixer's last product fills the rows)
+            self.mixer.forward_into(ctx, into, h, entry.cache, entry.writes_cache)
+        else:
+            if into is not x:
+                into.zero_()
+            self.mixer.forward_add(ctx, into, h, entry.cache, entry.writes_cache)
         if self.feed_forward is not None:
             self.feed_forward.forward_add(ctx, into, h)
         if into is not x:

@@ -89,8 +89,7 @@ def attend(ctx, out, q, cache, tables, num_heads, kv_heads, dk, dv, scale, sinks
         ops.attention_kv_plain(out, q, cache, ctx.positions, ctx.token_segment, tables, num_heads, kv_heads, dk, dv,
                                ctx.page_size, scale, sinks, weights=weights, gate=gate, **sight)
         return
-    plain_sight = not sight and gate is None
-    portions = ctx.extra[f"attention_kv.portions.{ops.attention_kv_rows(dk, dv, num_heads // kv_heads, weights, plain_sight)}"]
+    portions = ctx.extra[f"attention_kv.portions.{ops.attention_kv_rows(dk, dv, num_heads // kv_heads, weights)}"]
     singles = ctx.extra["attention_kv.singles"]
     if portions.shape[0]:
         ops.attention_kv_bf16(out, q, cache, portions, 0, tables, num_heads, kv_heads, dk, dv, ctx.page_size, scale, sinks,
@@ -104,7 +103,8 @@ def attend(ctx, out, q, cache, tables, num_heads, kv_heads, dk, dv, scale, sinks
             pooled = span // sight["pool"] if sight.get("pool") else 0
             tiles = min(tiles, -(-sight["window"] // _KEY_TILE) + 1 + -(-pooled // _KEY_TILE))
         units = kv_heads * -(-(num_heads // kv_heads) // _ROWS)
-        splits = max(1, min(tiles // 4, _WAVES_WANTED // (count * units), _MOST_SPLITS))
+        # (a split walks four tiles at least of keys and values of 256 dims together, and fewer of larger ones)
+        splits = max(1, min(tiles // max(1, 1024 // (dk + dv)), _WAVES_WANTED // (count * units), _MOST_SPLITS))
         partial = None
         if splits > 1:
             partial = ctx.workspace.flat("attention_kv.partial", ops.attention_kv_partial_words(count, num_heads, dv, splits),
@@ -150,11 +150,9 @@ class _KvMixer(Mixer):
         if self.position is not None:
             self.position.prepare(info.num_positions, info.device)
 
-    plain_sight = True        # False in a mixer whose calls name a window, pooled blocks, a cap or a gate
-
     def plan(self, plan):
         if self.matrix:
-            plan_items(plan, ops.attention_kv_rows(*self.kernel_sizes, self.weights, self.plain_sight))
+            plan_items(plan, ops.attention_kv_rows(*self.kernel_sizes, self.weights))
 
     def forward_add(self, ctx, x, h, cache_layer: int, writes_cache: bool):
         y = ctx.rows("mixer.rows_out", self.hidden, torch.float32)
@@ -344,7 +342,6 @@ class LatentAttention(_KvMixer):
         self.matrix = (self._matrix(self.dk_abs, self.dv_abs, self.num_heads * self.dk_abs, self.num_heads * self.dv_abs)
                        and self.down_width % 8 == 0 and self.q_rank % 8 == 0)
         self.sight = dict(window=self.window) if self.window else None
-        self.plain_sight = not self.window
 
     def tensor_specs(self):
         n, H = self.names, self.num_heads
@@ -461,7 +458,6 @@ class WindowAttention(_KvMixer):
         self.kernel_sizes = (self.dk, self.dv, self.num_heads // self.kv_heads)
         self.matrix = self._matrix(self.dk, self.dv, self.q_width, self.out_width)
         self.sight = dict(window=self.window, pool=self.pool, softcap=self.softcap, sections=self.sections)
-        self.plain_sight = False
 
     def tensor_specs(self):
         n = self.names

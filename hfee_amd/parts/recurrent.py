@@ -264,6 +264,12 @@ class Retention(_StateMixer):
             self.position.prepare(info.num_positions, info.device)
 
     def forward_add(self, ctx, x, h, cache_layer: int, writes_cache: bool):
+        self._run(ctx, x, h, add=True)
+
+    def forward_into(self, ctx, out, h, cache_layer: int, writes_cache: bool):
+        self._run(ctx, out, h, add=False)
+
+    def _run(self, ctx, x, h, add: bool):
         hn = h.tensor() if isinstance(h, LazyNorm) else h
         H, D, V = self.heads, self.dim, self.vdim
         rows, lengths, slots = self._segments(ctx)
@@ -283,7 +289,7 @@ class Retention(_StateMixer):
                         decay_per_head=True)
         gated = ctx.rows("retention.out", self.v_width)
         ops.head_norm_gate(gated, o, proj[:, self.at_g:], self.norm_weight, H, V, self.norm_eps, "silu")
-        product(ctx, x, gated, self.w_o, self.w_o_tiles, add=True)
+        product(ctx, x, gated, self.w_o, self.w_o_tiles, add=add)
 
 
 @register_mixer("state_space")

@@ -78,7 +78,7 @@ def windowed_definition(q, k, v, gate, scale, window, pool, cap):
 @pytest.mark.parametrize("H,G,dk,dv,window,pool,cap,gated", [
     (4, 2, 32, 16, 19, 5, 4.0, True), (3, 3, 10, 12, 7, 1, 0.0, False), (8, 2, 64, 64, 100, 7, 20.0, True),
     (2, 1, 16, 48, 5, 11, 0.0, True), (6, 2, 96, 96, 40, 12, 30.0, True), (4, 4, 32, 32, 33, 0, 0.0, False),
-    (4, 1, 96, 64, 0, 0, 0.0, False)])
+    (4, 1, 96, 64, 0, 0, 0.0, False), (8, 2, 32, 32, 50, 0, 0.0, False), (16, 1, 48, 32, 21, 0, 0.0, False)])
 def test_attention_over_a_window_with_pooled_blocks(dtype, H, G, dk, dv, window, pool, cap, gated):
     """Two sequences side by side, written in portions whose edges fall inside pages, windows and blocks, read
     by portions and by single tokens (plain, and where the sizes allow on the matrix cores, the single tokens'
@@ -115,7 +115,6 @@ def test_attention_over_a_window_with_pooled_blocks(dtype, H, G, dk, dv, window,
     bt = i32(tables)
     matrix = dtype == "bfloat16" and ops.attention_kv_sizes_fit(dk, dv)
     sight = dict(window=window, pool=pool if window else 0, softcap=cap, sections=sections)
-    plain_sight = not window and not cap and not gated
     # the values as the cache holds them: normed a head, rounded
     eps = 1e-5
     vn = [(v.double() / torch.sqrt((v.double() ** 2).mean(-1, keepdim=True) + eps)).to(dt).double() for v in vs]
@@ -140,7 +139,7 @@ def test_attention_over_a_window_with_pooled_blocks(dtype, H, G, dk, dv, window,
         ops.attention_kv_plain(out, q, cache, positions, token_segment, tab, H, G, dk, dv, 16, scale, gate=gate, **sight)
         outs = [out]
         if matrix:
-            rows_most = ops.attention_kv_rows(dk, dv, H // G, "softmax", plain_sight)
+            rows_most = ops.attention_kv_rows(dk, dv, H // G, "softmax")
             portions, singles, row = [], [], 0
             for i, (s, n) in enumerate(segs):
                 if n > 1:
