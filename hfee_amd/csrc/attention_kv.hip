@@ -187,7 +187,7 @@ __global__ __launch_bounds__(256) void rotate_norm_write_kernel(
 }
 
 // ---------------------------------------------------------------- pooled blocks
-// One wave a (token, key/value head): a token at the last position of a block of `pool` positions
+// One wave a (token, key/value head, 64 of the key's and value's dims): a token at the last position of a block of `pool` positions
 // (position % pool == pool - 1) leaves the block's key and value in the pooled section under the
 // block's number: the means of the block's keys and values as the cache holds them, summed in the
 // order of the positions in float32.  Every other token's wave has nothing to do.  Runs behind the
@@ -196,9 +196,11 @@ template <typename T>
 __global__ __launch_bounds__(256) void kv_pool_write_kernel(
     T* __restrict__ cache, KvLayout lay, int pool, int64_t pool_offset, const int* __restrict__ positions,
     const int* __restrict__ token_segment, const int* __restrict__ block_tables, int bt_stride, int n) {
+  const int parts = (lay.dk + lay.dv + 63) >> 6;
   const int64_t item = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  if (item >= (int64_t)n * lay.kv_heads) return;
-  const int t = (int)(item / lay.kv_heads), g = (int)(item % lay.kv_heads), lane = threadIdx.x & 63;
+  if (item >= (int64_t)n * lay.kv_heads * parts) return;
+  const int part_of_row = (int)(item % parts), lane = threadIdx.x & 63;
+  const int t = (int)(item / parts / lay.kv_heads), g = (int)(item / parts % lay.kv_heads);
   const int pos = positions[t];
   if (pos % pool != pool - 1) return;
   const int b = pos / pool;
@@ -206,7 +208,8 @@ __global__ __launch_bounds__(256) void kv_pool_write_kernel(
   T* pooled = cache + pool_offset;
   const int to_page = bt[b >> lay.page_shift], to_slot = b & (lay.page_size - 1);
   const float share = 1.0f / (float)pool;
-  for (int d = lane; d < lay.dk + lay.dv; d += 64) {
+  const int d = part_of_row * 64 + lane;
+  if (d < lay.dk + lay.dv) {
     float sum = 0.f;
     for (int j0 = pos - pool + 1; j0 <= pos; j0 += 8) {       // eight loads on their way at a time, added in order
       T part[8];
@@ -494,7 +497,7 @@ HFEE_API int hfee_kv_pool_write(void* cache, int dtype, int pool, const int* pos
   if (n == 0) return 0;
   KvLayout lay;
   if (make_kv_layout(&lay, kv_heads, dk, dv, page_size, 2)) return 1;
-  const int64_t items = (int64_t)n * kv_heads;
+  const int64_t items = (int64_t)n * kv_heads * ((dk + dv + 63) / 64);
   HFEE_REQUIRE((items + 3) / 4 <= 0x7fffffff, "kv_pool_write: too much work for one launch");
   const int64_t pool_offset = (int64_t)page_size * (dk + dv);
 #define LAUNCH(T)                                                                                                    \

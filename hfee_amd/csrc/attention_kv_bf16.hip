@@ -597,9 +597,9 @@ __global__ __launch_bounds__(256) void attention_kv_shared_kernel(
   }
 }
 
-// joins the splits of a single token's heads: one wave per (item, head).  Lane sp holds split sp's
-// maximum and sum (at most 64 splits), the weights of the splits come from one reduction over the
-// wave, and the value dims are then summed over the splits in their order, lanes over the dims.
+// joins the splits of a single token's heads: one wave per (item, head, 64 value dims).  Lane sp holds split
+// sp's maximum and sum (at most 64 splits), the weights of the splits come from one reduction over the
+// wave, and the wave's value dims are then summed over the splits in their order, lanes over the dims.
 __global__ __launch_bounds__(64) void attention_kv_join_kernel(
     bf16_t* __restrict__ out, int64_t ld_out, const int* __restrict__ items, const float* __restrict__ partial,
     int splits, int num_heads, const float* __restrict__ sinks, const bf16_t* __restrict__ gate, int64_t ld_gate) {
@@ -615,12 +615,11 @@ __global__ __launch_bounds__(64) void attention_kv_join_kernel(
   const float lsum = wave_sum(my_l * my_w) + (!SIGMOID && sinks != nullptr ? exp2f(sk - m) : 0.f);
   float inv = SIGMOID ? 1.0f : 1.0f / lsum;
   if (gate != nullptr) inv *= 1.0f / (1.0f + __expf(-bf16_to_float(gate[(int64_t)token * ld_gate + head])));
-  for (int d = lane; d < DV; d += 64) {
-    float o = 0.f;
+  const int d = blockIdx.z * 64 + lane;
+  float o = 0.f;
 #pragma unroll 8
-    for (int sp = 0; sp < splits; ++sp) o = fmaf(pr[sp * kPartial + 4 + d], __shfl(my_w, sp, 64), o);
-    out[(int64_t)token * ld_out + (int64_t)head * DV + d] = float_to_bf16(o * inv);
-  }
+  for (int sp = 0; sp < splits; ++sp) o = fmaf(d < DV ? pr[sp * kPartial + 4 + d] : 0.f, __shfl(my_w, sp, 64), o);
+  if (d < DV) out[(int64_t)token * ld_out + (int64_t)head * DV + d] = float_to_bf16(o * inv);
 }
 
 }  // namespace
@@ -700,7 +699,7 @@ HFEE_API int hfee_attention_kv_bf16(void* out, int64_t ld_out, const void* q, in
         sight, (const bf16_t*)gate, ld_gate);
   HFEE_CHECK_LAUNCH("attention_kv_bf16");
   if (splits > 1) {
-    attention_kv_join_kernel<<<dim3(num_items, num_heads), 64, 0, stream>>>((bf16_t*)out, ld_out, items, partial,
+    attention_kv_join_kernel<<<dim3(num_items, num_heads, (DV + 63) / 64), 64, 0, stream>>>((bf16_t*)out, ld_out, items, partial,
                                                                             splits, num_heads, sinks,
                                                                             (const bf16_t*)gate, ld_gate);
     HFEE_CHECK_LAUNCH("attention_kv_bf16 join");

@@ -200,3 +200,48 @@ HFEE_API int hfee_scaled_add(float* x, const float* y, float a, const float* y2,
   HFEE_CHECK_LAUNCH("scaled_add");
   return 0;
 }
+
+namespace {
+// A workgroup a row: x += a y, then next = x / sqrt(mean(x^2) + eps) * w in the engine's dtype (the norm of
+// whatever reads the stream next).  A thread keeps its elements of the new row in registers between the sum
+// and the scaling where the row has at most 256 x 16 of them; a longer row is read again.
+constexpr int kAddNormKeep = 16;
+
+template <typename T>
+__global__ __launch_bounds__(256) void scaled_add_norm_kernel(float* __restrict__ x, const float* __restrict__ y, float a,
+                                                              T* __restrict__ next, const float* __restrict__ w, float eps,
+                                                              int width) {
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  float* xr = x + row * width;
+  const float* yr = y + row * width;
+  T* nr = next + row * width;
+  float kept[kAddNormKeep];
+  float ss = 0.f;
+  int i = 0;
+  for (int c = threadIdx.x; c < width; c += 256, ++i) {
+    const float v = fmaf(a, yr[c], xr[c]);
+    xr[c] = v;
+    if (i < kAddNormKeep) kept[i] = v;
+    ss = fmaf(v, v, ss);
+  }
+  const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+  i = 0;
+  for (int c = threadIdx.x; c < width; c += 256, ++i) {
+    const float v = i < kAddNormKeep ? kept[i] : xr[c];
+    nr[c] = from_float<T>(v * inv * w[c]);
+  }
+}
+}  // namespace
+
+// x (float32 [n, width], contiguous) += a y; next ([n, width] in dtype) = the RMS norm of the new rows with weight w.
+HFEE_API int hfee_scaled_add_norm(float* x, const float* y, float a, void* next, int dtype, const float* w, float eps, int n,
+                                  int width, hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && width > 0 && y != nullptr && next != nullptr && w != nullptr && eps >= 0.f, "scaled_add_norm: bad arguments");
+  if (n == 0) return 0;
+  if (dtype == 0) scaled_add_norm_kernel<float><<<n, 256, 0, stream>>>(x, y, a, (float*)next, w, eps, width);
+  else if (dtype == 1) scaled_add_norm_kernel<bf16_t><<<n, 256, 0, stream>>>(x, y, a, (bf16_t*)next, w, eps, width);
+  else return fail("scaled_add_norm: unknown dtype %d", dtype);
+  HFEE_CHECK_LAUNCH("scaled_add_norm");
+  return 0;
+}

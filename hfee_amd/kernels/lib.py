@@ -69,6 +69,7 @@ _CORE_SIGNATURES = {
     "hfee_router_topk": [P, L, I, I, I, P, P, I, P, P],
     "hfee_add_table_rows": [P, I, I, P, I, P, P],
     "hfee_scaled_add": [P, P, F, P, F, L, P],
+    "hfee_scaled_add_norm": [P, P, F, P, I, P, F, I, I, P],
     "hfee_gated_norm_add": [P, P, P, F, F, P, I, L, P, P, F, P, I, P, F, I, I, P],
     "hfee_head_norm_gate": [P, L, P, L, P, L, I, P, I, I, F, I, I, P],
     "hfee_moe_grouped": [P, L, P, L, P, P, P, P, P, P, P, F, I, I, I, I, I, P, P, P, P, P, P],

@@ -1085,6 +1085,19 @@ def scaled_add(x, y, a: float = 1.0, y2=None, b: float = 1.0):
     lib.core().call("hfee_scaled_add", _ptr(x), _ptr(y), float(a), _ptr(y2), float(b), x.numel(), _stream())
 
 
+def scaled_add_norm(x, y, a: float, next_out, next_weight, next_eps: float):
+    """x += a * y (float32, contiguous, one shape), and next_out (the engine's dtype, contiguous) = the RMS norm of
+    the new rows, x / sqrt(mean(x^2) + next_eps) * next_weight (float32 [width])."""
+    _gpu(x, y, next_out, next_weight)
+    _check(x.dtype == y.dtype == torch.float32 and x.is_contiguous() and y.is_contiguous() and x.shape == y.shape and x.dim() == 2,
+           "scaled_add_norm: contiguous float32 rows x and y of one shape")
+    _check(next_out.is_contiguous() and next_out.shape == x.shape, "scaled_add_norm: next_out like x")
+    _check(next_weight.dtype == torch.float32 and next_weight.is_contiguous() and next_weight.numel() == x.shape[1],
+           "scaled_add_norm: next_weight float32 [width]")
+    lib.core().call("hfee_scaled_add_norm", _ptr(x), _ptr(y), float(a), _ptr(next_out), _dt(next_out), _ptr(next_weight),
+                    float(next_eps), x.shape[0], x.shape[1], _stream())
+
+
 def gated_norm_add(x, y, weight, eps: float, y2=None, scales=(1.0, 1.0), gate=None, gate_bias=None, next_out=None,
                    next_weight=None, next_eps: float = 0.0):
     """With v = (scales[0] * y + scales[1] * y2) * sigmoid(gate + gate_bias) (y2 and the gate optional):

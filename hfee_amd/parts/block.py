@@ -18,7 +18,7 @@ returns).
 x += mixer(h) + feed_forward(h).  Both add their last product straight into the float32 stream, the
 mixer first; a layer may have no feed-forward.  With the parameter `residual_scale` = m the layer adds
 m * (mixer(h) + feed_forward(h)): the sub-layers then add into float32 rows of their own, which join the
-stream in one launch.
+stream in one launch that also makes the next layer's norm (or the head's) where that is an RMS norm.
 """
 from __future__ import annotations
 
@@ -252,9 +252,13 @@ class ParallelBlock(Part):
         for p in self._own():
             p.bind(tensors)
 
-    def forward(self, ctx, x, entry):
-        h = ctx.rows("block.normed", self.hidden)
-        self.norm.forward(ctx, h, x)
+    chains_norms = True
+
+    def begin(self, ctx, x):
+        return LazyNorm(ctx, self.norm, x)
+
+    def forward(self, ctx, x, entry, h_in=None, h_next=None):
+        h = (h_in if h_in is not None else self.begin(ctx, x)).tensor()
         into = x
         if self.residual_scale != 1.0:
             into = ctx.rows("block.sublayer_rows", self.hidden, torch.float32)
@@ -267,4 +271,10 @@ class ParallelBlock(Part):
         if self.feed_forward is not None:
             self.feed_forward.forward_add(ctx, into, h)
         if into is not x:
-            ops.scaled_add(x, into, self.residual_scale)
+            form = h_next.norm.fused_form_f32() if h_next is not None and hasattr(h_next.norm, "fused_form_f32") else None
+            if form is not None and h_next._tensor is None and h_next.pending is None:
+                out = ctx.rows("block.normed", self.hidden)
+                ops.scaled_add_norm(x, into, self.residual_scale, out, form[0], form[1])
+                h_next._tensor = out
+            else:
+                ops.scaled_add(x, into, self.residual_scale)
