@@ -279,7 +279,7 @@ def saposun_config(size: dict, layers: int, vocab: int = 32000) -> dict:
     heads = d // 256
     ret = {"type": "retention", "mixer": {"heads": heads, "dim": 128, "vdim": 256, "rot": {"base": 500000.0, "dims": 128},
                                           "decay": [1.0 - 2.0 ** (-5 - 3 * i / max(1, heads - 1)) for i in range(heads)]}}
-    att = {"type": "attention", "mixer": {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "softcap": 30.0,
+    att = {"type": "attention", "mixer": {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "softcap": 50.0,
                                           "conv": 4, "mask": {"size": 1024, "pool": 16}, "rot": {"base": 500000.0, "dims": hd}}}
     moe = {"kind": "moe", "expert": {"ff": size["expert_ff"]}, "router": {"experts": 16, "top": 2}}
     out = []
@@ -288,7 +288,7 @@ def saposun_config(size: dict, layers: int, vocab: int = 32000) -> dict:
         if i % 6 == 3:          # every other latent layer reads the keys of the one three layers before it
             layer = {"type": "latent_attention", "mixer": dict(latent, kv_from=i - 3)}
         out.append(dict(layer, mlp=moe))
-    return {"architecture": "Saposun", "vocab": vocab, "width": d, "norm": {"eps": 1e-5}, "residual_mult": 0.3,
+    return {"architecture": "Saposun", "vocab": vocab, "width": d, "norm": {"eps": 1e-5}, "residual_mult": 0.5,
             "max_positions": 4096, "layers": out}
 
 

@@ -204,11 +204,12 @@ HFEE_API int hfee_scaled_add(float* x, const float* y, float a, const float* y2,
 namespace {
 // A workgroup a row: x += a y, then next = x / sqrt(mean(x^2) + eps) * w in the engine's dtype (the norm of
 // whatever reads the stream next).  A thread keeps its elements of the new row in registers between the sum
-// and the scaling where the row has at most 256 x 16 of them; a longer row is read again.
+// and the scaling where it has at most 16 of them; a longer row is read again.  256 threads a row, 1,024
+// where the rows are few (a row's time is then the chain of its loads).
 constexpr int kAddNormKeep = 16;
 
 template <typename T>
-__global__ __launch_bounds__(256) void scaled_add_norm_kernel(float* __restrict__ x, const float* __restrict__ y, float a,
+__global__ __launch_bounds__(1024) void scaled_add_norm_kernel(float* __restrict__ x, const float* __restrict__ y, float a,
                                                               T* __restrict__ next, const float* __restrict__ w, float eps,
                                                               int width) {
   __shared__ float scratch[16];
@@ -219,7 +220,7 @@ __global__ __launch_bounds__(256) void scaled_add_norm_kernel(float* __restrict_
   float kept[kAddNormKeep];
   float ss = 0.f;
   int i = 0;
-  for (int c = threadIdx.x; c < width; c += 256, ++i) {
+  for (int c = threadIdx.x; c < width; c += blockDim.x, ++i) {
     const float v = fmaf(a, yr[c], xr[c]);
     xr[c] = v;
     if (i < kAddNormKeep) kept[i] = v;
@@ -227,7 +228,7 @@ __global__ __launch_bounds__(256) void scaled_add_norm_kernel(float* __restrict_
   }
   const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
   i = 0;
-  for (int c = threadIdx.x; c < width; c += 256, ++i) {
+  for (int c = threadIdx.x; c < width; c += blockDim.x, ++i) {
     const float v = i < kAddNormKeep ? kept[i] : xr[c];
     nr[c] = from_float<T>(v * inv * w[c]);
   }
@@ -239,8 +240,9 @@ HFEE_API int hfee_scaled_add_norm(float* x, const float* y, float a, void* next,
                                   int width, hipStream_t stream) {
   HFEE_REQUIRE(n >= 0 && width > 0 && y != nullptr && next != nullptr && w != nullptr && eps >= 0.f, "scaled_add_norm: bad arguments");
   if (n == 0) return 0;
-  if (dtype == 0) scaled_add_norm_kernel<float><<<n, 256, 0, stream>>>(x, y, a, (float*)next, w, eps, width);
-  else if (dtype == 1) scaled_add_norm_kernel<bf16_t><<<n, 256, 0, stream>>>(x, y, a, (bf16_t*)next, w, eps, width);
+  const int threads = n <= 64 && width > 1024 ? 1024 : 256;
+  if (dtype == 0) scaled_add_norm_kernel<float><<<n, threads, 0, stream>>>(x, y, a, (float*)next, w, eps, width);
+  else if (dtype == 1) scaled_add_norm_kernel<bf16_t><<<n, threads, 0, stream>>>(x, y, a, (bf16_t*)next, w, eps, width);
   else return fail("scaled_add_norm: unknown dtype %d", dtype);
   HFEE_CHECK_LAUNCH("scaled_add_norm");
   return 0;

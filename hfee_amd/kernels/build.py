@@ -58,7 +58,7 @@ def attention_mix_fits(heads: int, dim: int) -> bool:
 # the pairs that `build_all` compiles: those of the tests and of bench.py's comparison (a model with
 # other sizes compiles its own at first use)
 ATTENTION_KV_SIZES = ((32, 16), (64, 32), (96, 64), (48, 32), (16, 48), (112, 96), (64, 64), (160, 128), (128, 128), (576, 512),
-                      (32, 32), (80, 64), (96, 96))
+                      (32, 32), (80, 64))
 # the same for the kernels without a softmax
 ATTENTION_KV_SIGMOID_SIZES = ((16, 32), (16, 48), (32, 64), (128, 128))
 

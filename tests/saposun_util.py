@@ -89,7 +89,7 @@ P_C = config(60, 48, 1e-6, 0.7, [
 ])
 # larger, for prompts of hundreds of tokens: windows over several pages and tiles, hundreds of pooled blocks' worth of
 # tokens, experts of sizes that the grouped kernels take
-P_D = config(500, 128, 1e-6, 0.3, [
+P_D = config(500, 128, 1e-6, 0.4, [
     moe(latent(8, 16, 16, 32, 48, 64, 0.15, window=70), 64, 8, 2),
     moe(retention(4, 32, 32, (0.95, 0.98, 0.99, 0.999), rot_dims=32), 64, 8, 2),
     moe(attention(8, 2, 64, 64, 0.12, window=100, pool=7, conv=4, softcap=20.0, rot_dims=64), 96, 8, 2),
@@ -106,6 +106,10 @@ SINGLE = {
     "attention": config(50, 48, 1e-6, 0.5, [bare(attention(4, 2, 12, 6, 0.4, window=10, pool=3, conv=3, softcap=3.0, rot_dims=6))]),
     "attention without anything": config(50, 64, 1e-6, 2.0, [bare(attention(4, 4, 32, 32, 0.2))]),
     "moe": config(50, 48, 1e-6, 0.5, [moe(retention(1, 4, 4, (0.5,)), 20, 7, 3)]),
+    # a width that is a multiple of nothing, a convolution of one tap (no state), two layers so that the scaled sum
+    # makes the next layer's norm
+    "odd width": config(61, 58, 1e-6, 0.25, [moe(attention(2, 1, 14, 10, 0.3, window=9, pool=4, conv=1, rot_dims=14), 9, 3, 2),
+                                              moe(latent(2, 5, 6, 7, 9, 11, 0.3, window=4), 9, 3, 3)]),
 }
 
 

@@ -77,7 +77,7 @@ def windowed_definition(q, k, v, gate, scale, window, pool, cap):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("H,G,dk,dv,window,pool,cap,gated", [
     (4, 2, 32, 16, 19, 5, 4.0, True), (3, 3, 10, 12, 7, 1, 0.0, False), (8, 2, 64, 64, 100, 7, 20.0, True),
-    (2, 1, 16, 48, 5, 11, 0.0, True), (6, 2, 96, 96, 40, 12, 30.0, True), (4, 4, 32, 32, 33, 0, 0.0, False),
+    (2, 1, 16, 48, 5, 11, 0.0, True), (6, 2, 80, 64, 45, 9, 25.0, True), (4, 4, 32, 32, 33, 0, 0.0, False),
     (4, 1, 96, 64, 0, 0, 0.0, False), (8, 2, 32, 32, 50, 0, 0.0, False), (16, 1, 48, 32, 21, 0, 0.0, False)])
 def test_attention_over_a_window_with_pooled_blocks(dtype, H, G, dk, dv, window, pool, cap, gated):
     """Two sequences side by side, written in portions whose edges fall inside pages, windows and blocks, read
@@ -288,6 +288,19 @@ def test_the_router_adds_its_correction_to_the_choice_only(n, E, top):
     ops.router_topk(chosen, weights, logits.cuda(), top, score="softmax", correction=big.cuda())
     assert (chosen[:, 0] == E - 1).all()
     assert su.rel(weights[:, 0].double().cpu(), scores[:, E - 1]) < 1e-6
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n,width", [(8, 4096), (100, 72), (3, 5000), (70, 1024), (1, 58)])
+def test_the_scaled_sum_with_the_next_norm(dtype, n, width):
+    from hfee_amd.kernels import ops
+    g = torch.Generator().manual_seed(n + width)
+    x, y, w = torch.randn(n, width, generator=g), torch.randn(n, width, generator=g), torch.rand(width, generator=g) + 0.5
+    got_x, nxt = x.clone().cuda(), torch.zeros(n, width, dtype=DT[dtype], device="cuda")
+    ops.scaled_add_norm(got_x, y.cuda(), 0.3, nxt, w.cuda(), 1e-5)
+    want_x = x.double() + 0.3 * y.double()
+    assert su.rel(got_x.double().cpu(), want_x) < 1e-6
+    assert su.rel(nxt.double().cpu(), ps.rms_norm(want_x, w.double(), 1e-5)) < (2e-6 if dtype == "float32" else 1e-2)
 
 
 # ------------------------------------------------------------------ the whole model
