@@ -27,12 +27,21 @@ def _rope(head_dim: int, rot, pairing: str):
     return PositionSpec("rope", params(head_dim=head_dim, rotary_dim=rot.dims, theta=rot.base, scaling=None, pairing=pairing))
 
 
-def _mixer(cfg: SaposunConfig, m) -> MixerSpec:
+def _kept_positions(cfg: SaposunConfig, i: int) -> int:
+    """How many positions the cache layer that latent layer i reads must keep: the widest window of the layers
+    that read it (0: one of them sees every earlier position, so every token is kept)."""
+    source = cfg.layers[i].mixer.kv_from if cfg.layers[i].mixer.kv_from is not None else i
+    windows = [l.mixer.window for k, l in enumerate(cfg.layers)
+               if isinstance(l.mixer, WindowLatentConfig) and (k == source or l.mixer.kv_from == source)]
+    return 0 if not all(windows) else max(windows)
+
+
+def _mixer(cfg: SaposunConfig, m, i: int = 0) -> MixerSpec:
     if isinstance(m, WindowLatentConfig):
         return MixerSpec("latent_attention", params(
             hidden=cfg.width, num_heads=m.heads, plain_dim=m.dim, rotated_dim=m.rot_dim, value_dim=m.vdim,
             q_rank=m.q_rank, kv_rank=m.kv_rank, scale=m.scale, norm_eps=cfg.norm_eps, window=m.window,
-            own_keys=m.kv_from is None,
+            own_keys=m.kv_from is None, cache_window=_kept_positions(cfg, i),
             names=(("q_down", "dq"), ("q_norm", "dq.norm"), ("q_up", "uq"), ("kv_down", "dkv"),
                    ("kv_norm", "dkv.norm"), ("k_up", "uk"), ("v_up", "uv"), ("o", "o"))),
             position=_rope(m.rot_dim, m.rot, "interleaved"))
@@ -64,7 +73,7 @@ def _feed_forward(cfg: SaposunConfig, mlp):
 def saposun_model_spec(cfg: SaposunConfig) -> ModelSpec:
     norm = NormSpec("rmsnorm", cfg.width, cfg.norm_eps)
     layers = tuple(
-        LayerSpec(arrangement="parallel", hidden=cfg.width, mixer=_mixer(cfg, layer.mixer),
+        LayerSpec(arrangement="parallel", hidden=cfg.width, mixer=_mixer(cfg, layer.mixer, i),
                   feed_forward=_feed_forward(cfg, layer.mlp), mixer_norm=norm, feed_forward_norm=norm, prefix=f"l{i}.",
                   names=(("mixer", "mix."), ("feed_forward", "mlp."), ("mixer_norm", "norm1")),
                   params=params(residual_scale=cfg.residual_mult))

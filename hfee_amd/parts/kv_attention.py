@@ -19,7 +19,9 @@ size rank + rotated dims), the weighted sum is taken over the latents themselves
 rank), and W_uv,h is applied to the result.  Prompt portions and single tokens then run the same
 kernels, and a token's logits do not depend on how its prompt was cut.
 
-With `window` a query sees the last `window` positions only, itself included.  With `own_keys` False the
+With `window` a query sees the last `window` positions only, itself included; with `cache_window` (at least
+the window of every layer that reads the cache layer) the layer's pages form a "window" group of the cache
+manager, which takes back the pages that every such window has passed.  With `own_keys` False the
 layer has no W_dkv: it reads the latent and the rotated key part that another layer of the same latent
 size, rotated part and rotation keeps (the schedule names that layer's cache), with its own W_uk and W_uv.
 The rotation's pairs may be (i, i + half) or (2i, 2i + 1): the score is a sum over the rotated dims, so for
@@ -327,6 +329,9 @@ class LatentAttention(_KvMixer):
         self.scale = float(spec.get("scale", (self.plain + self.rotated) ** -0.5))
         self.eps = float(spec.get("norm_eps", 1e-6))
         self.window = int(spec.get("window", 0))
+        self.cache_window = int(spec.get("cache_window", 0) or 0)
+        if self.cache_window and not 0 < self.window <= self.cache_window:
+            raise ValueError(f"a cache that keeps {self.cache_window} positions cannot serve a window of {self.window or 'all'}")
         self.own_keys = bool(spec.get("own_keys", True))
         self.position = lookup("position", spec.position.kind)(spec.position) if spec.position else None
         if self.position is not None and self.position.rotary_dim != self.rotated:
@@ -379,6 +384,8 @@ class LatentAttention(_KvMixer):
         self.w_down_tiles, self.w_q_up_tiles, self.w_o_tiles = tiles_of(self.dtype, self.w_down, self.w_q_up, self.w_o)
 
     def cache_spec(self):
+        if self.cache_window:
+            return CacheNeed("window", (1, self.dk_abs + self.dv_abs), self.cache_window, layout=_LAYOUT)
         return CacheNeed("full", (1, self.dk_abs + self.dv_abs), 0, layout=_LAYOUT)
 
     def key_layout(self):

@@ -433,6 +433,28 @@ def test_a_slot_that_is_used_again_starts_from_nothing(folders, plain_rows, name
     compare(got, want, "float32", f"{name}: one slot for all")
 
 
+def test_a_window_gives_back_the_pages_it_has_passed(folders, plain_rows):
+    """The latent layers' cache is a window group of the manager: a request of 150 tokens holds the pages of its
+    widest window and no more, whether it came in portions or token by token, and its logits are the plain ones."""
+    from hfee_amd.trace_replay import Replayer
+    reqs, want = plain_rows("latent", "float32", [150])
+    toks = reqs["r0"]
+    rep = Replayer(folders[("latent", "float32")], "float32", 192, max_requests=2)
+    groups = rep.engine.cache.groups
+    assert [g.kind for g in groups] == ["window"] and groups[0].window == 6
+    got, fed = {}, 0
+    for n in [40, 3, 2, 50] + [1] * 55:
+        rows = rep.step([("r0", toks[fed:fed + n], list(range(n)))])
+        got.update({("r0", fed + i): rows[i] for i in range(n)})
+        fed += n
+        held = [p for p in rep.engine.cache.get("r0").tables[0] if p >= 0]
+        assert len(held) <= 2, (fed, held)          # a window of 6 positions touches two pages of 16 at most
+        rep.engine.cache.check()
+    compare(got, want, "float32", "a window group")
+    rep.engine.release("r0")
+    assert not rep.engine.cache.requests
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(folders, dtype):
     """300 single tokens after a short prompt: decode steps replayed from captured graphs, across page borders,
