@@ -390,7 +390,8 @@ def design_point(cj: dict, batch: int, steps: int, warmup: int) -> dict:
     step_bytes = weight_bytes + batch * context_read * bytes_per_token(engine.groups, torch.bfloat16) + 2 * batch * state_bytes
     for elements, w, p, own in windows:      # (a layer behind a window reads the window and the pooled blocks, not the context;
         reads = min(context_read, w) + (context_read / p if p else 0)      # one that reads another layer's keys has no cache layer)
-        step_bytes -= batch * 2 * elements * ((context_read * (2 if p else 1) if own else 0) - reads)
+        pooled_entries = context_read / p if p else 0                    # (the pooled blocks' group is counted by its share already)
+        step_bytes -= batch * 2 * elements * ((context_read + pooled_entries if own else 0) - reads)
     for r in list(sched.running):
         sched.cancel(r.request_id)
     while sched.has_work():

@@ -9,7 +9,9 @@ cache group, a block table (page ids by position // page_size) and one state slo
 Groups: layers whose caches have the same needs share a group and a page id
 addresses the same place in each of the group's layers.  A "full" group keeps every
 key; a "window" group keeps the last `window` keys, and pages that the window has
-passed go back to the pool at commit time.  Pages come back when a request is
+passed go back to the pool at commit time.  A group with `every` = P > 1 grows by one
+entry every P tokens (a pooled block of P tokens, say): a request of n tokens holds
+ceil(n / P) entries of it, in ceil(ceil(n / P) / page_size) pages.  Pages come back when a request is
 released and are handed out again at once (last freed, first reused).
 
 Prefixes kept between requests.  The reference leaves a finished request's cache in its
@@ -53,12 +55,15 @@ class CacheGroupSpec:
     cache_layers: tuple       # ids of the cache layers in this group
     window: int = 0           # keys kept per token for kind == "window"
     layout: str = ""
+    every: int = 1            # tokens an entry: the group grows by one entry every `every` tokens
 
     def __post_init__(self):
         if self.kind not in ("full", "window"):
             raise CacheError(f"unknown cache group kind {self.kind!r}")
         if self.kind == "window" and self.window <= 0:
             raise CacheError("a window group needs a positive window")
+        if int(self.every) < 1 or (self.every > 1 and self.kind != "full"):
+            raise CacheError("a group grows by one entry every `every` >= 1 tokens, and only a full group by fewer than one a token")
         if not self.token_shape or any(int(n) < 1 for n in self.token_shape):
             raise CacheError(f"a token must add at least one element to a cache layer, got {self.token_shape!r}")
 
@@ -158,7 +163,7 @@ class CacheManager:
         self.max_requests = max_requests
         self._free_slots = list(range(max_requests - 1, -1, -1))
         self.requests: dict = {}
-        if keep_prefixes and any(g.kind != "full" for g in self.groups):
+        if keep_prefixes and any(g.kind != "full" or g.every != 1 for g in self.groups):
             raise CacheError("prefixes can be kept only where every cache group keeps every token")
         self.keep_prefixes = bool(keep_prefixes) and bool(self.groups)
         # digest of the tokens up to a page's end -> (the page in every group, the page's own tokens);
@@ -259,20 +264,36 @@ class CacheManager:
         return len(self._free_slots)
 
     # --------------------------------------------------------------- pages
-    def _blocks_for(self, length: int) -> int:
-        return (length + self.page_size - 1) // self.page_size
+    def _blocks_for(self, length: int, group: int | None = None) -> int:
+        """Pages that `length` tokens take in a group (in a group that holds every token, without one)."""
+        every = 1 if group is None else self.groups[group].every
+        entries = (length + every - 1) // every
+        return (entries + self.page_size - 1) // self.page_size
 
     def pages_needed(self, request_id, n_new: int) -> list:
         """Pages each group would have to take so that positions
         length .. length + n_new - 1 have a place."""
         rc = self.get(request_id)
-        want = self._blocks_for(rc.length + n_new)
-        return [max(0, want - len(t)) for t in rc.tables]
+        return [max(0, self._blocks_for(rc.length + n_new, g) - len(t)) for g, t in enumerate(rc.tables)]
 
     def pages_for_tokens(self, n_tokens: int) -> list:
         """Pages per group that a fresh request of n_tokens holds at most at one time
         when it is run in one portion."""
-        return [self._blocks_for(n_tokens)] * len(self.groups)
+        return [self._blocks_for(n_tokens, g) for g in range(len(self.groups))]
+
+    def room(self, request_id) -> int:
+        """How many more tokens of the request its pages and the free pages can hold (the least over the groups;
+        a page of a group that grows every few tokens holds that many times a page's tokens)."""
+        rc = self.get(request_id)
+        room = None
+        for spec, table, pool in zip(self.groups, rc.tables, self.pools):
+            r = (len(table) + pool.num_free) * self.page_size * spec.every - rc.length
+            room = r if room is None else min(room, r)
+        return max(room or 0, 0)
+
+    def free_tokens(self):
+        """Tokens that the free pages hold (the least over the groups); None without any group."""
+        return min((p.num_free * self.page_size * g.every for g, p in zip(self.groups, self.pools)), default=None)
 
     def can_reserve(self, request_id, n_new: int) -> bool:
         return all(need <= pool.num_free for need, pool in zip(self.pages_needed(request_id, n_new), self.pools))
@@ -300,7 +321,7 @@ class CacheManager:
         """The step has written n_new tokens: advance the length and return the
         pages that a window has passed."""
         rc = self.get(request_id)
-        if any(self._blocks_for(rc.length + n_new) > len(t) for t in rc.tables):
+        if any(self._blocks_for(rc.length + n_new, g) > len(t) for g, t in enumerate(rc.tables)):
             raise CacheError(f"request {request_id!r}: commit of {n_new} tokens beyond the reserved pages")
         rc.length += n_new
         for g, spec in enumerate(self.groups):
@@ -325,9 +346,9 @@ class CacheManager:
         rc = self.get(request_id)
         if not 0 <= length <= rc.length:
             raise CacheError(f"cannot truncate request {request_id!r} from {rc.length} to {length}")
-        keep = self._blocks_for(length)
         for g, spec in enumerate(self.groups):
             table = rc.tables[g]
+            keep = self._blocks_for(length, g)
             if spec.kind == "window" and length > 0 and any(
                     table[b] < 0 for b in range(max(0, (length - spec.window) // self.page_size), min(keep, len(table)))):
                 raise CacheError("a window group has already released pages this truncation needs")

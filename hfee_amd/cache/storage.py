@@ -72,5 +72,6 @@ class CacheStorage:
 
 
 def bytes_per_token(groups, dtype: torch.dtype) -> int:
+    """What a token adds to the cache (a group that grows by an entry every `every` tokens: its share)."""
     size = torch.empty((), dtype=dtype).element_size()
-    return sum(len(g.cache_layers) * g.token_elements * size for g in groups)
+    return sum(-(-len(g.cache_layers) * g.token_elements * size // g.every) for g in groups)

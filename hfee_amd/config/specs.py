@@ -72,11 +72,16 @@ class CacheNeed:
     that a token adds to the layer (keys and values of attention: (2, kv_heads, head_dim); a
     latent vector: (width,)); how they are arranged inside a page is the part's own affair
     (`layout` names it: two parts may share a cache layer only if they agree on it).  Cache
-    layers with equal needs share a group of pages."""
+    layers with equal needs share a group of pages.  `every` > 1: the layer grows by one entry every
+    `every` tokens (entry b belongs to the tokens b * every .. b * every + every - 1: a pooled block, a
+    summary), and a request of n tokens holds ceil(n / every) entries of it.  A part that needs two kinds
+    of growing memory answers `cache_spec()` with a tuple of needs; the first is the cache layer that the
+    schedule names, need k > 0 lives under the cache layer (that layer, k)."""
     kind: str                 # "full": every token is kept; "window": the last `window` tokens
     token_shape: tuple
     window: int = 0
     layout: str = ""
+    every: int = 1
 
 
 @dataclass(frozen=True)

@@ -32,9 +32,7 @@ struct KvLayout {
   }
 };
 
-// A page may hold `sections` such parts a head, one behind the other: the tokens' keys and values first,
-// then (a second section) one pooled key and value for every block of tokens, under the block's number.
-inline int make_kv_layout(KvLayout* out, int kv_heads, int dk, int dv, int page_size, int sections = 1) {
+inline int make_kv_layout(KvLayout* out, int kv_heads, int dk, int dv, int page_size) {
   if (page_size < 16 || (page_size & (page_size - 1)) != 0)
     return fail("page_size must be a power of two >= 16, got %d", page_size);
   if (kv_heads < 1 || dk < 1 || dv < 1) return fail("bad cache shape: kv_heads %d dk %d dv %d", kv_heads, dk, dv);
@@ -42,8 +40,7 @@ inline int make_kv_layout(KvLayout* out, int kv_heads, int dk, int dv, int page_
   out->dk = dk;
   out->dv = dv;
   out->page_size = page_size;
-  if (sections < 1 || sections > 2) return fail("a page holds one or two sections a head, not %d", sections);
-  out->head_stride = (int64_t)sections * page_size * (dk + dv);
+  out->head_stride = (int64_t)page_size * (dk + dv);
   out->page_stride = (int64_t)kv_heads * out->head_stride;
   int s = 0;
   while ((1 << s) < page_size) ++s;
@@ -53,12 +50,15 @@ inline int make_kv_layout(KvLayout* out, int kv_heads, int dk, int dv, int page_
 
 // What a query at position p sees: the keys first_key(p) .. p, and the pooled blocks 0 .. pooled_blocks(p) - 1
 // (block b holds the positions b * pool .. b * pool + pool - 1 and is seen once all of them have left the
-// window: b * pool + pool - 1 <= p - window).
+// window: b * pool + pool - 1 <= p - window).  The pooled blocks are a cache layer of their own, of the same
+// sizes and the same arrangement a page as the tokens', with block tables of its own: block b is its entry b.
 struct KeySight {
-  int window;            // 0: every earlier position
-  int pool;              // 0: no pooled blocks
-  float softcap;         // 0: scores as they are
-  int64_t pool_offset;   // elements from a (page, head)'s first section to its pooled one
+  int window;               // 0: every earlier position
+  int pool;                 // 0: no pooled blocks
+  float softcap;            // 0: scores as they are
+  const void* pooled;       // the pooled blocks' cache layer
+  const int* pool_tables;   // its block tables, a row a segment as the tokens' have
+  int pool_bt_stride;
 
   __host__ __device__ __forceinline__ int first_key(int p) const { return window > 0 && p - window + 1 > 0 ? p - window + 1 : 0; }
   __host__ __device__ __forceinline__ int pooled_blocks(int p) const {
@@ -67,13 +67,17 @@ struct KeySight {
   __device__ __forceinline__ float capped(float s) const { return softcap > 0.f ? softcap * tanhf(s / softcap) : s; }
 };
 
-inline int make_key_sight(KeySight* out, int window, int pool, float softcap, int sections, int page_size, int dk, int dv) {
+inline int make_key_sight(KeySight* out, int window, int pool, float softcap, const void* pooled, const int* pool_tables,
+                          int pool_bt_stride) {
   if (window < 0 || pool < 0 || !(softcap >= 0.f)) return fail("bad window %d, pool %d or softcap %f", window, pool, (double)softcap);
-  if (pool > 0 && sections != 2) return fail("pooled blocks live in a page's second section");
+  if (pool > 0 && window > 0 && (pooled == nullptr || pool_tables == nullptr))
+    return fail("pooled blocks need their cache layer and its block tables");
   out->window = window;
-  out->pool = pool;
+  out->pool = window > 0 ? pool : 0;
   out->softcap = softcap;
-  out->pool_offset = (int64_t)page_size * (dk + dv);
+  out->pooled = pooled;
+  out->pool_tables = pool_tables;
+  out->pool_bt_stride = pool_bt_stride;
   return 0;
 }
 

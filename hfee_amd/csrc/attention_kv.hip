@@ -188,14 +188,15 @@ __global__ __launch_bounds__(256) void rotate_norm_write_kernel(
 
 // ---------------------------------------------------------------- pooled blocks
 // One wave a (token, key/value head, 64 of the key's and value's dims): a token at the last position of a block of `pool` positions
-// (position % pool == pool - 1) leaves the block's key and value in the pooled section under the
-// block's number: the means of the block's keys and values as the cache holds them, summed in the
+// (position % pool == pool - 1) leaves the block's key and value in the pooled blocks' cache layer under
+// the block's number: the means of the block's keys and values as the cache holds them, summed in the
 // order of the positions in float32.  Every other token's wave has nothing to do.  Runs behind the
 // launch that wrote the step's keys and values.
 template <typename T>
 __global__ __launch_bounds__(256) void kv_pool_write_kernel(
-    T* __restrict__ cache, KvLayout lay, int pool, int64_t pool_offset, const int* __restrict__ positions,
-    const int* __restrict__ token_segment, const int* __restrict__ block_tables, int bt_stride, int n) {
+    const T* __restrict__ cache, T* __restrict__ pooled, KvLayout lay, int pool, const int* __restrict__ positions,
+    const int* __restrict__ token_segment, const int* __restrict__ block_tables, int bt_stride,
+    const int* __restrict__ pool_tables, int pool_bt_stride, int n) {
   const int parts = (lay.dk + lay.dv + 63) >> 6;
   const int64_t item = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (item >= (int64_t)n * lay.kv_heads * parts) return;
@@ -205,8 +206,8 @@ __global__ __launch_bounds__(256) void kv_pool_write_kernel(
   if (pos % pool != pool - 1) return;
   const int b = pos / pool;
   const int* bt = block_tables + (int64_t)token_segment[t] * bt_stride;
-  T* pooled = cache + pool_offset;
-  const int to_page = bt[b >> lay.page_shift], to_slot = b & (lay.page_size - 1);
+  const int* pbt = pool_tables + (int64_t)token_segment[t] * pool_bt_stride;
+  const int to_page = pbt[b >> lay.page_shift], to_slot = b & (lay.page_size - 1);
   const float share = 1.0f / (float)pool;
   const int d = part_of_row * 64 + lane;
   if (d < lay.dk + lay.dv) {
@@ -255,14 +256,15 @@ __global__ __launch_bounds__(64) void attention_kv_plain_kernel(
   const int pos = positions[t];
   const int* bt = block_tables + (int64_t)token_segment[t] * bt_stride;
   const int first = sight.first_key(pos), blocks = sight.pooled_blocks(pos);
-  const T* pooled = cache + sight.pool_offset;
+  const T* pooled = static_cast<const T*>(sight.pooled);
+  const int* pbt = sight.pool_tables + (int64_t)token_segment[t] * sight.pool_bt_stride;
 
   for (int d = lane; d < dk; d += 64) qs[d] = to_float<T>(q[(int64_t)t * ldq + (int64_t)h * dk + d]);
   __syncthreads();
 
-  // the score of entry j of a section (the tokens' or the pooled blocks'), as the softmax takes it
-  auto score = [&](const T* section, int j) {
-    const T* kr = section + lay.key_offset(bt[j >> lay.page_shift], kvh, j & (lay.page_size - 1), 0);
+  // the score of entry j of a layer (the tokens' or the pooled blocks'), as the softmax takes it
+  auto score = [&](const T* section, const int* table, int j) {
+    const T* kr = section + lay.key_offset(table[j >> lay.page_shift], kvh, j & (lay.page_size - 1), 0);
     float s = 0.f;
     for (int d = 0; d < dk; ++d) s = fmaf(qs[d], to_float<T>(kr[d]), s);
     return sight.capped(s * scale);
@@ -270,10 +272,10 @@ __global__ __launch_bounds__(64) void attention_kv_plain_kernel(
   float m = -INFINITY;
   if (weighting == 0) {
     for (int base = 0; base < blocks; base += 64)
-      if (base + lane < blocks) m = fmaxf(m, score(pooled, base + lane));
+      if (base + lane < blocks) m = fmaxf(m, score(pooled, pbt, base + lane));
     for (int base = first & ~63; base <= pos; base += 64) {
       const int j = base + lane;
-      if (j >= first && j <= pos) m = fmaxf(m, score(cache, j));
+      if (j >= first && j <= pos) m = fmaxf(m, score(cache, bt, j));
     }
   }
   m = wave_max(m);
@@ -285,13 +287,13 @@ __global__ __launch_bounds__(64) void attention_kv_plain_kernel(
   float o[kMaxDvPerLane];
 #pragma unroll
   for (int r = 0; r < kMaxDvPerLane; ++r) o[r] = 0.f;
-  // entries [from, to] of a section, 64 at a time from a multiple of 64: lane (j mod 64) owns entry j
-  auto walk = [&](const T* section, int from, int to) {
+  // entries [from, to] of a layer, 64 at a time from a multiple of 64: lane (j mod 64) owns entry j
+  auto walk = [&](const T* section, const int* table, int from, int to) {
     for (int base = from & ~63; base <= to; base += 64) {
       const int j = base + lane;
       float e = 0.f;
       if (j >= from && j <= to) {
-        const float s = score(section, j);
+        const float s = score(section, table, j);
         e = weighting == 0 ? expf(s - m) : 1.0f / (1.0f + expf(-(s + sink)));
         lsum += e;
       }
@@ -301,7 +303,7 @@ __global__ __launch_bounds__(64) void attention_kv_plain_kernel(
       const int je = min(base + 63, to);
       for (int jj = max(base, from); jj <= je; ++jj) {
         const float w = es[jj - base];
-        const int page = bt[jj >> lay.page_shift], slot = jj & (lay.page_size - 1);
+        const int page = table[jj >> lay.page_shift], slot = jj & (lay.page_size - 1);
 #pragma unroll
         for (int r = 0; r < kMaxDvPerLane; ++r) {
           const int d = lane + 64 * r;
@@ -310,8 +312,8 @@ __global__ __launch_bounds__(64) void attention_kv_plain_kernel(
       }
     }
   };
-  if (blocks > 0) walk(pooled, 0, blocks - 1);
-  walk(cache, first, pos);
+  if (blocks > 0) walk(pooled, pbt, 0, blocks - 1);
+  walk(cache, bt, first, pos);
   lsum = wave_sum(lsum);
   if (has_sink) lsum += expf(sink - m);
   if (weighting != 0) lsum = 1.0f;
@@ -461,7 +463,7 @@ HFEE_API int hfee_rotate_norm_write(void* q_out, int64_t ldqo, const float* q, i
                                     int64_t ldk, const float* v, int64_t ldv, float value_eps, int dtype, const float* cos_t,
                                     const float* sin_t, int half, int table_positions, int max_position,
                                     const int* positions, const int* token_segment, const int* block_tables, int bt_stride,
-                                    void* cache, int kv_heads, int dk, int dv, int page_size, int sections, int n,
+                                    void* cache, int kv_heads, int dk, int dv, int page_size, int n,
                                     hipStream_t stream) {
   HFEE_REQUIRE(n >= 0 && num_heads > 0 && q != nullptr && q_out != nullptr, "rotate_norm_write: bad arguments");
   if (n == 0) return 0;
@@ -470,7 +472,7 @@ HFEE_API int hfee_rotate_norm_write(void* q_out, int64_t ldqo, const float* q, i
   HFEE_REQUIRE(half == 0 || max_position < table_positions,
                "rotate_norm_write: position %d is beyond the rotation tables of %d positions", max_position, table_positions);
   KvLayout lay;
-  if (make_kv_layout(&lay, kv_heads, dk, dv, page_size, sections)) return 1;
+  if (make_kv_layout(&lay, kv_heads, dk, dv, page_size)) return 1;
   HFEE_REQUIRE(ldq >= (int64_t)num_heads * dk && ldqo >= (int64_t)num_heads * dk, "rotate_norm_write: q rows too short");
   if (k != nullptr) {
     HFEE_REQUIRE(v != nullptr && cache != nullptr && token_segment != nullptr && block_tables != nullptr,
@@ -490,19 +492,19 @@ HFEE_API int hfee_rotate_norm_write(void* q_out, int64_t ldqo, const float* q, i
   return 0;
 }
 
-HFEE_API int hfee_kv_pool_write(void* cache, int dtype, int pool, const int* positions, const int* token_segment,
-                                const int* block_tables, int bt_stride, int kv_heads, int dk, int dv, int page_size, int n,
-                                hipStream_t stream) {
-  HFEE_REQUIRE(n >= 0 && pool >= 1 && cache != nullptr, "kv_pool_write: bad arguments");
+HFEE_API int hfee_kv_pool_write(const void* cache, void* pooled, int dtype, int pool, const int* positions,
+                                const int* token_segment, const int* block_tables, int bt_stride, const int* pool_tables,
+                                int pool_bt_stride, int kv_heads, int dk, int dv, int page_size, int n, hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && pool >= 1 && cache != nullptr && pooled != nullptr && block_tables != nullptr && pool_tables != nullptr,
+               "kv_pool_write: bad arguments");
   if (n == 0) return 0;
   KvLayout lay;
-  if (make_kv_layout(&lay, kv_heads, dk, dv, page_size, 2)) return 1;
+  if (make_kv_layout(&lay, kv_heads, dk, dv, page_size)) return 1;
   const int64_t items = (int64_t)n * kv_heads * ((dk + dv + 63) / 64);
   HFEE_REQUIRE((items + 3) / 4 <= 0x7fffffff, "kv_pool_write: too much work for one launch");
-  const int64_t pool_offset = (int64_t)page_size * (dk + dv);
 #define LAUNCH(T)                                                                                                    \
-  kv_pool_write_kernel<T><<<(unsigned)((items + 3) / 4), 256, 0, stream>>>((T*)cache, lay, pool, pool_offset, positions,  \
-      token_segment, block_tables, bt_stride, n)
+  kv_pool_write_kernel<T><<<(unsigned)((items + 3) / 4), 256, 0, stream>>>((const T*)cache, (T*)pooled, lay, pool, positions, \
+      token_segment, block_tables, bt_stride, pool_tables, pool_bt_stride, n)
   if (dtype == 0) LAUNCH(float);
   else if (dtype == 1) LAUNCH(bf16_t);
   else return fail("kv_pool_write: unknown dtype %d", dtype);
@@ -515,11 +517,11 @@ HFEE_API int hfee_attention_kv_plain(void* out, int64_t ld_out, const void* q, i
                                      int dtype, const int* positions, const int* token_segment,
                                      const int* block_tables, int bt_stride, int num_heads, int kv_heads, int dk,
                                      int dv, int page_size, float scale, const float* sinks, int weighting, int window,
-                                     int pool, float softcap, int sections, const void* gate, int64_t ld_gate, int n,
-                                     hipStream_t stream) {
+                                     int pool, float softcap, const void* pooled, const int* pool_tables, int pool_bt_stride,
+                                     const void* gate, int64_t ld_gate, int n, hipStream_t stream) {
   HFEE_REQUIRE(n >= 0, "attention_kv_plain: bad token count");
   KeySight sight;
-  if (make_key_sight(&sight, window, pool, softcap, sections, page_size, dk, dv)) return 1;
+  if (make_key_sight(&sight, window, pool, softcap, pooled, pool_tables, pool_bt_stride)) return 1;
   HFEE_REQUIRE(gate == nullptr || ld_gate >= num_heads, "attention_kv_plain: the gates' rows are too short");
   HFEE_REQUIRE(weighting == 0 || weighting == 1, "attention_kv_plain: the weights are a softmax's (0) or sigmoids (1)");
   if (n == 0) return 0;
@@ -530,7 +532,7 @@ HFEE_API int hfee_attention_kv_plain(void* out, int64_t ld_out, const void* q, i
   HFEE_REQUIRE(num_heads <= 65535, "attention_kv_plain: too many heads");
   HFEE_REQUIRE(ldq >= (int64_t)num_heads * dk && ld_out >= (int64_t)num_heads * dv, "attention_kv_plain: q/out row too short");
   KvLayout lay;
-  if (make_kv_layout(&lay, kv_heads, dk, dv, page_size, sections)) return 1;
+  if (make_kv_layout(&lay, kv_heads, dk, dv, page_size)) return 1;
   dim3 grid(n, num_heads);
   const size_t lds = (dk + 64) * sizeof(float);
   if (dtype == 0)

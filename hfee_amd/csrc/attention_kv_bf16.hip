@@ -18,9 +18,9 @@
 //
 // A query may see less than every earlier key (`KeySight`, attention_kv.h): the last `window` positions only,
 // and beside them one pooled key and value for every block of `pool` positions that lies wholly before the
-// window (the second section of the pages, under the block's number); a score may be capped as
+// window (a cache layer of their own with block tables of its own, under the block's number); a score may be capped as
 // cap * tanh(score / cap); a head's result may be multiplied by sigmoid of a gate.  The kernel then walks
-// the tiles of the pooled section that any of its rows sees, and after them the token tiles from the one
+// the tiles of the pooled layer that any of its rows sees, and after them the token tiles from the one
 // that holds the first key of its first row's window; a key weighs where it lies within its row's bounds.
 //
 // Compiled with -DHFEE_KV_WEIGHTS=1 there is no softmax: a visible key weighs sigmoid(score + b_h), b_h a
@@ -215,7 +215,7 @@ __global__ __launch_bounds__(256) void attention_kv_kernel(
     for (int vb = 0; vb < VBLOCKS; ++vb) acc[b][vb] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  // the tiles to walk: those of the pooled section that any row sees, then the token tiles from the first
+  // the tiles to walk: those of the pooled layer that any row sees, then the token tiles from the first
   // key of the first row's window on (without a window or pooled blocks: the token tiles from the first)
   const int pool_tiles = (sight.pooled_blocks(max_pos) + 31) >> 5;
   const int tile_lo = sight.first_key(pos0) >> 5;
@@ -224,7 +224,9 @@ __global__ __launch_bounds__(256) void attention_kv_kernel(
   const int tile_begin = split * per_split, tile_end = min(ntiles, tile_begin + per_split);
   const int last_block = max_pos >> lay.page_shift;
   const int slot_mask = lay.page_size - 1;
-  const bf16_t* const pooled = cache + sight.pool_offset;
+  const bf16_t* const pooled = static_cast<const bf16_t*>(sight.pooled);
+  const int* const pbt = sight.pool_tables + (int64_t)items[item * 4 + 3] * sight.pool_bt_stride;
+  const int last_pool_block = max(sight.pooled_blocks(max_pos) - 1, 0) >> lay.page_shift;
 
   // the key operands of a tile: lane (r, g) holds dims 8g .. 8g+7 of every step of key r of each of the
   // tile's two blocks of 16 keys; `values` gets where the lane's value columns of the two blocks begin
@@ -234,7 +236,7 @@ __global__ __launch_bounds__(256) void attention_kv_kernel(
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
       const int jb = (tile << 5) + kb * 16;
-      const int page = bt[min(jb >> lay.page_shift, last_block)];
+      const int page = walked < pool_tiles ? pbt[min(jb >> lay.page_shift, last_pool_block)] : bt[min(jb >> lay.page_shift, last_block)];
       const int slot0 = jb & slot_mask;
       const bf16_t* kr = section + lay.key_offset(page, kvh, slot0 + r, g * 8);
       values[kb] = section + lay.values_of(page, kvh) + slot0 + g * 4;
@@ -250,7 +252,7 @@ __global__ __launch_bounds__(256) void attention_kv_kernel(
     const bf16_t* section = walked < pool_tiles ? pooled : cache;
     const int tile = walked < pool_tiles ? walked : tile_lo + walked - pool_tiles;
     const int jb = (tile << 5) + kb * 16;
-    const int page = bt[min(jb >> lay.page_shift, last_block)];
+    const int page = walked < pool_tiles ? pbt[min(jb >> lay.page_shift, last_pool_block)] : bt[min(jb >> lay.page_shift, last_block)];
     const int slot0 = jb & slot_mask;
     values = section + lay.values_of(page, kvh) + slot0 + g * 4;
     Operand one;
@@ -440,14 +442,16 @@ __global__ __launch_bounds__(256) void attention_kv_shared_kernel(
     for (int vb = 0; vb < VBLOCKS; ++vb) acc[b][vb] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
   const int max_pos = pos0 + rows - 1;
-  // the tiles to walk: those of the pooled section that any row sees, then the token tiles from the first key
+  // the tiles to walk: those of the pooled layer that any row sees, then the token tiles from the first key
   // of the first row's window on
   const int pool_tiles = (sight.pooled_blocks(max_pos) + 31) >> 5;
   const int tile_lo = sight.first_key(pos0) >> 5;
   const int ntiles = pool_tiles + (max_pos >> 5) + 1 - tile_lo;
   const int last_block = max_pos >> lay.page_shift;
   const int slot_mask = lay.page_size - 1;
-  const bf16_t* const pooled = cache + sight.pool_offset;
+  const bf16_t* const pooled = static_cast<const bf16_t*>(sight.pooled);
+  const int* const pbt = sight.pool_tables + (int64_t)items[item * 4 + 3] * sight.pool_bt_stride;
+  const int last_pool_block = max(sight.pooled_blocks(max_pos) - 1, 0) >> lay.page_shift;
 
   // two sets of registers for the chunks on their way, where that is few registers: a tile is then
   // asked for two tiles before it is multiplied (memory takes longer than one tile's products)
@@ -461,7 +465,7 @@ __global__ __launch_bounds__(256) void attention_kv_shared_kernel(
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
       const int jb = (tile << 5) + kb * 16;
-      const int page = bt[min(jb >> lay.page_shift, last_block)];
+      const int page = walked < pool_tiles ? pbt[min(jb >> lay.page_shift, last_pool_block)] : bt[min(jb >> lay.page_shift, last_block)];
       keys[kb] = section + lay.key_offset(page, kvh, jb & slot_mask, 0);
       values[kb] = section + lay.values_of(page, kvh) + (jb & slot_mask);
     }
@@ -646,11 +650,13 @@ HFEE_API int hfee_attention_kv_bf16(void* out, int64_t ld_out, const void* q, in
                                     const int* items, int num_items, int mode, const int* block_tables,
                                     int bt_stride, int num_heads, int kv_heads, int page_size, float scale,
                                     const float* sinks, float* partial, int64_t partial_words, int splits,
-                                    int window, int pool, float softcap, int sections, const void* gate,
+                                    int window, int pool, float softcap, const void* pooled, const int* pool_tables,
+                                    int pool_bt_stride, const void* gate,
                                     int64_t ld_gate, hipStream_t stream) {
   HFEE_REQUIRE(num_items >= 0, "attention_kv_bf16: bad item count");
   KeySight sight;
-  if (make_key_sight(&sight, window, pool, softcap, sections, page_size, DK, DV)) return 1;
+  if (make_key_sight(&sight, window, pool, softcap, pooled, pool_tables, pool_bt_stride)) return 1;
+  HFEE_REQUIRE(pooled == nullptr || (uintptr_t)pooled % 16 == 0, "attention_kv_bf16: the pooled layer must be aligned for vector access");
   HFEE_REQUIRE(gate == nullptr || ld_gate >= num_heads, "attention_kv_bf16: the gates' rows are too short");
   if (num_items == 0) return 0;
   HFEE_REQUIRE(mode == 0 || mode == 1, "attention_kv_bf16: mode is 0 (portions) or 1 (single tokens)");
@@ -665,7 +671,7 @@ HFEE_API int hfee_attention_kv_bf16(void* out, int64_t ld_out, const void* q, in
                partial_words >= hfee_attention_kv_bf16_partial(num_items, num_heads, splits)),
                "attention_kv_bf16: the partial results need more room");
   KvLayout lay;
-  if (make_kv_layout(&lay, kv_heads, DK, DV, page_size, sections)) return 1;
+  if (make_kv_layout(&lay, kv_heads, DK, DV, page_size)) return 1;
   const int hpg = num_heads / kv_heads;
   const int64_t units = mode == 0 ? num_heads : (int64_t)kv_heads * ((hpg + 15) / 16);
   const int64_t waves = (int64_t)num_items * splits * units;

@@ -75,21 +75,27 @@ class Model:
         return out
 
     # ---- cache
+    def _needs_of(self, layer: int) -> tuple:
+        """The needs of a block's cache layers: none, one, or several (the first is the cache layer that the
+        schedule names, need k > 0 the cache layer (that layer, k))."""
+        need = self.blocks[layer].cache_spec()
+        return () if need is None else tuple(need) if isinstance(need, (tuple, list)) else (need,)
+
     def cache_groups(self):
         """Cache layers with the same needs share a group.  A cache layer's needs are
         those of the block that writes it (a block answers for the part of it that uses
         the cache)."""
         needs: dict = {}
         for e in self.schedule:
-            need = self.blocks[e.layer].cache_spec()
-            if need is None:
+            if not e.writes_cache:
                 continue
-            if e.writes_cache:
-                if e.cache in needs and needs[e.cache] != need:
-                    raise ValueError(f"cache layer {e.cache} is written by layers with different needs")
-                needs[e.cache] = need
+            for k, need in enumerate(self._needs_of(e.layer)):
+                key = e.cache if k == 0 else (e.cache, k)
+                if key in needs and needs[key] != need:
+                    raise ValueError(f"cache layer {key} is written by layers with different needs")
+                needs[key] = need
         for e in self.schedule:
-            need = self.blocks[e.layer].cache_spec()
+            need = next(iter(self._needs_of(e.layer)), None)
             if need is not None and not e.writes_cache:
                 if e.cache not in needs:
                     raise ValueError(f"layer {e.layer} reads cache layer {e.cache}, which no layer writes")
@@ -101,10 +107,10 @@ class Model:
                     raise ValueError(f"layer {e.layer} cannot read cache layer {e.cache}: its keys are laid out "
                                      f"differently from those that layer {writer.layer} writes")
         by_need: dict = {}
-        for layer, need in sorted(needs.items()):
+        for layer, need in sorted(needs.items(), key=lambda kv: kv[0] if isinstance(kv[0], tuple) else (kv[0], 0)):
             by_need.setdefault(need, []).append(layer)
         return [CacheGroupSpec(kind=n.kind, token_shape=tuple(n.token_shape), window=n.window, layout=n.layout,
-                               cache_layers=tuple(layers))
+                               every=n.every, cache_layers=tuple(layers))
                 for n, layers in by_need.items()]
 
     def state_specs(self):

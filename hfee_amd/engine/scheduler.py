@@ -144,13 +144,7 @@ class Scheduler:
     # ------------------------------------------------------------------ pages
     def _room(self, request: Request) -> int:
         """How many more tokens of `request` the free pages can hold."""
-        rc = self.cache.get(request.request_id)
-        ps = self.cache.page_size
-        room = None
-        for table, pool in zip(rc.tables, self.cache.pools):
-            r = len(table) * ps - rc.length + pool.num_free * ps
-            room = r if room is None else min(room, r)
-        return max(room or 0, 0)
+        return self.cache.room(request.request_id)
 
     def _comes_back_with(self, request: Request) -> int:
         """Free tokens that a preempted request waits for while others run: room for all it has
@@ -261,8 +255,7 @@ class Scheduler:
                 continue          # preempted while an older request was served
             if budget == 0:
                 break
-            rc = self.cache.requests[r.request_id]
-            if any(len(t) * ps <= rc.length for t in rc.tables):      # its next token starts a new page
+            if any(self.cache.pages_needed(r.request_id, 1)):      # its next token starts a new page
                 while self._room(r) < 1 and self.running[-1] is not r:
                     victim = self.running[-1]          # always younger than r
                     batch = [b for b in batch if b[0] is not victim]
@@ -295,7 +288,7 @@ class Scheduler:
         while self.waiting and len(self.running) < self.max_num_seqs and self.cache.num_free_slots > 0 and budget > 0:
             r = self.waiting[0]
             first = min(len(r.feed), budget)
-            free_tokens = min(p.num_free for p in self.cache.pools) * self.cache.page_size if self.cache.pools else first
+            free_tokens = self.cache.free_tokens() if self.cache.pools else first
             if free_tokens < min(first, self.cache.page_size) and self.running:
                 break                      # wait until pages come back
             if r.request_id in self._preempted_now:

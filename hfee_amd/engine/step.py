@@ -83,10 +83,14 @@ class Engine:
             num_pages = capacity.choose_pages(wanted, at_most, *self._memory(), self._workspace_estimate(),
                                               page_size * bytes_per_token(self.groups, self.dtype),
                                               self._state_bytes())
+        if not isinstance(num_pages, (list, tuple)) and any(g.every > 1 for g in self.groups):
+            # (a group that grows by an entry every few tokens holds that share of the pages, and a page more a request)
+            num_pages = [num_pages if g.every == 1 else -(-num_pages // g.every) + max_requests for g in self.groups]
         self.num_pages = num_pages
         # (a finished request's full pages wait for a request that begins alike: only where every
         # group keeps every token and no part has state that cannot be cut back)
-        keep_prefixes = bool(keep_prefixes) and all(g.kind == "full" for g in self.groups) and not model.state_specs()
+        keep_prefixes = (bool(keep_prefixes) and all(g.kind == "full" and g.every == 1 for g in self.groups)
+                         and not model.state_specs())
         self.cache = CacheManager(self.groups, page_size, num_pages, max_requests, keep_prefixes=keep_prefixes)
         self.storage = CacheStorage(self.groups, page_size, num_pages, max_requests, self.dtype, self.device)
         self.workspace = Workspace(max_batch_tokens, self.device)

@@ -48,9 +48,9 @@ _CORE_SIGNATURES = {
     "hfee_read_stream": [P, L, P, I, I, P],
     "hfee_mfma_loop": [P, I, I, P],
     "hfee_kv_write": [P, L, I, I, I, P, L, I, P, L, P, I, P, I, P, P, P, I, P, P, I, I, I, P, I, I, I, I, I, P],
-    "hfee_attention_kv_plain": [P, L, P, L, P, I, P, P, P, I, I, I, I, I, I, F, P, I, I, I, F, I, P, L, I, P],
-    "hfee_rotate_norm_write": [P, L, P, L, I, P, L, P, L, F, I, P, P, I, I, I, P, P, P, I, P, I, I, I, I, I, I, P],
-    "hfee_kv_pool_write": [P, I, I, P, P, P, I, I, I, I, I, I, P],
+    "hfee_attention_kv_plain": [P, L, P, L, P, I, P, P, P, I, I, I, I, I, I, F, P, I, I, I, F, P, P, I, P, L, I, P],
+    "hfee_rotate_norm_write": [P, L, P, L, I, P, L, P, L, F, I, P, P, I, I, I, P, P, P, I, P, I, I, I, I, I, P],
+    "hfee_kv_pool_write": [P, P, I, I, P, P, P, I, P, I, I, I, I, I, I, P],
     "hfee_rotate_rows": [P, L, P, L, I, P, P, P, I, I, I, I, I, I, F, I, P],
     "hfee_qk_norm_write": [P, L, I, P, L, P, L, I, P, P, F, F, I, P, P, P, I, P, I, I, I, I, I, P],
     "hfee_head_linear": [P, L, L, P, L, L, P, I, I, I, I, I, I, P],
@@ -83,7 +83,7 @@ _ATTENTION_KV_SIGNATURES = {
     "hfee_attention_kv_bf16_dv": [],
     "hfee_attention_kv_bf16_weights": [],
     "hfee_attention_kv_bf16_rows": [I],
-    "hfee_attention_kv_bf16": [P, L, P, L, P, P, I, I, P, I, I, I, I, F, P, P, L, I, I, I, F, I, P, L, P],
+    "hfee_attention_kv_bf16": [P, L, P, L, P, P, I, I, P, I, I, I, I, F, P, P, L, I, I, I, F, P, P, I, P, L, P],
 }
 
 _ATTENTION_MIX_SIGNATURES = {

@@ -792,10 +792,10 @@ def _qkv_rows(out, x, weight, q):
 
 # ------------------------------- attention with keys and values of sizes of their own, and a sink
 
-def _kv_cache(cache_layer, kv_heads, dk, dv, page_size, what, sections: int = 1):
+def _kv_cache(cache_layer, kv_heads, dk, dv, page_size, what):
     _check(cache_layer.is_contiguous() and cache_layer.dim() == 3 and
-           tuple(cache_layer.shape[1:]) == (kv_heads, sections * page_size * (dk + dv)),
-           f"{what}: the cache layer must be [pages, kv_heads, sections * page_size * (key size + value size)]")
+           tuple(cache_layer.shape[1:]) == (kv_heads, page_size * (dk + dv)),
+           f"{what}: the cache layer must be [pages, kv_heads, page_size * (key size + value size)]")
 
 
 def kv_write(q, k, v, positions, token_segment, block_tables, cos, sin, cache_layer, num_heads: int, kv_heads: int,
@@ -849,29 +849,40 @@ def kv_write(q, k, v, positions, token_segment, block_tables, cos, sin, cache_la
 KEY_WEIGHTS = {"softmax": 0, "sigmoid": 1}
 
 
-def _sight(window: int, pool: int, softcap: float, sections: int, what: str):
-    _check(window >= 0 and pool >= 0 and softcap >= 0 and sections in (1, 2), f"{what}: bad window, pool, softcap or sections")
-    _check(not pool or sections == 2, f"{what}: pooled blocks live in a page's second section")
+def _sight(window: int, pool: int, softcap: float, pooled, pool_tables, cache_layer, segments: int, what: str):
+    """(the pooled layer, its block tables, their row stride) for the entry points; pooled blocks are a cache layer of
+    the tokens' shape and dtype with block tables of its own, a row a segment."""
+    _check(window >= 0 and pool >= 0 and softcap >= 0, f"{what}: bad window, pool or softcap")
+    if not (pool and window):
+        return None, None, 0
+    _check(pooled is not None and pool_tables is not None, f"{what}: pooled blocks need their cache layer and its block tables")
+    _check(pooled.is_contiguous() and pooled.dtype == cache_layer.dtype and tuple(pooled.shape[1:]) == tuple(cache_layer.shape[1:]),
+           f"{what}: the pooled layer must have the tokens' page shape and dtype")
+    _check(pool_tables.dtype == torch.int32 and pool_tables.dim() == 2 and pool_tables.stride(1) == 1
+           and pool_tables.shape[0] >= segments, f"{what}: the pooled layer's block tables")
+    return pooled, pool_tables, pool_tables.stride(0)
 
 
 def attention_kv_plain(out, q, cache_layer, positions, token_segment, block_tables, num_heads: int, kv_heads: int,
                        dk: int, dv: int, page_size: int, scale: float, sinks=None, weights: str = "softmax",
-                       window: int = 0, pool: int = 0, softcap: float = 0.0, sections: int = 1, gate=None):
+                       window: int = 0, pool: int = 0, softcap: float = 0.0, pooled=None, pool_tables=None, gate=None):
     """One wave per (token, head), any sizes, both dtypes: token t of head h reads the keys
     0..pos of its sequence; `sinks` (float32 [num_heads] or None) joins the softmax's denominator.
     weights "sigmoid": no softmax, a key weighs sigmoid(score + sinks[head]) and nothing is normalized.
     window > 0: only the last `window` positions, the token's own included; pool > 0: also one key and
-    value (a page's second section, under the block's number) for every block of `pool` positions that lies
-    wholly before the window; softcap > 0: a score s counts as softcap * tanh(s / softcap).
+    value (entry b of the cache layer `pooled`, which has block tables of its own, `pool_tables`) for every
+    block b of `pool` positions that lies wholly before the window; softcap > 0: a score s counts as
+    softcap * tanh(s / softcap).
     gate ([n, num_heads] in the tensors' dtype): head h's result is multiplied by sigmoid(gate[t, h])."""
     _check(weights in KEY_WEIGHTS, f"attention_kv: the weights are {sorted(KEY_WEIGHTS)}, not {weights!r}")
-    _gpu(out, q, cache_layer, positions, token_segment, block_tables, sinks, gate)
+    _gpu(out, q, cache_layer, positions, token_segment, block_tables, sinks, gate, pooled, pool_tables)
     n, w, ldq = _rows2d(q, "attention_kv q")
     no, wo, ldo = _rows2d(out, "attention_kv out")
     _check(no == n and w == num_heads * dk and wo == num_heads * dv, "attention_kv: q/out shape")
     _check(q.dtype == out.dtype == cache_layer.dtype, "attention_kv: dtype mismatch")
-    _sight(window, pool, softcap, sections, "attention_kv")
-    _kv_cache(cache_layer, kv_heads, dk, dv, page_size, "attention_kv", sections)
+    _kv_cache(cache_layer, kv_heads, dk, dv, page_size, "attention_kv")
+    pooled, pool_tables, pool_stride = _sight(window, pool, softcap, pooled, pool_tables, cache_layer, block_tables.shape[0],
+                                              "attention_kv")
     _i32(positions, "attention_kv positions", n)
     _i32(token_segment, "attention_kv token_segment", n)
     _check(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.stride(1) == 1,
@@ -886,11 +897,12 @@ def attention_kv_plain(out, q, cache_layer, positions, token_segment, block_tabl
     lib.core().call("hfee_attention_kv_plain", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), _dt(q),
                     _ptr(positions), _ptr(token_segment), _ptr(block_tables), block_tables.stride(0),
                     num_heads, kv_heads, dk, dv, page_size, float(scale), _ptr(sinks), KEY_WEIGHTS[weights],
-                    int(window), int(pool), float(softcap), int(sections), _ptr(gate), ldg, n, _stream())
+                    int(window), int(pool), float(softcap), _ptr(pooled), _ptr(pool_tables), pool_stride, _ptr(gate), ldg, n,
+                    _stream())
 
 
 def rotate_norm_write(q_out, q, k, v, positions, token_segment, block_tables, cos, sin, cache_layer, num_heads: int,
-                      kv_heads: int, dk: int, dv: int, page_size: int, max_position: int, value_eps=None, sections: int = 1):
+                      kv_heads: int, dk: int, dv: int, page_size: int, max_position: int, value_eps=None):
     """From float32 projections (behind a short convolution): q ([n, num_heads * dk]) rotated into q_out (the
     cache's dtype), k rotated and v into the token's slot of `cache_layer`, v divided by its root mean square
     over each head where value_eps is a number.  The first 2 * half dims of a head are rotated, pairs
@@ -906,7 +918,7 @@ def rotate_norm_write(q_out, q, k, v, positions, token_segment, block_tables, co
         nv, wv, ldv = _f32rows(v, "rotate_norm_write v")
         _check(nk == nv == n and wk == kv_heads * dk and wv == kv_heads * dv and q_out.dtype == cache_layer.dtype,
                "rotate_norm_write: k/v shapes, or the cache's dtype")
-        _kv_cache(cache_layer, kv_heads, dk, dv, page_size, "rotate_norm_write", sections)
+        _kv_cache(cache_layer, kv_heads, dk, dv, page_size, "rotate_norm_write")
         _i32(token_segment, "rotate_norm_write token_segment", n)
         _check(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.stride(1) == 1,
                "rotate_norm_write: block tables")
@@ -920,24 +932,26 @@ def rotate_norm_write(q_out, q, k, v, positions, token_segment, block_tables, co
                     -1.0 if value_eps is None else float(value_eps), _dt(q_out), _ptr(cos), _ptr(sin), half, table_positions,
                     int(max_position), _ptr(positions), _ptr(token_segment if has_k else None),
                     _ptr(block_tables if has_k else None), block_tables.stride(0) if has_k else 0,
-                    _ptr(cache_layer if has_k else None), kv_heads, dk, dv, page_size, int(sections), n, _stream())
+                    _ptr(cache_layer if has_k else None), kv_heads, dk, dv, page_size, n, _stream())
 
 
-def kv_pool_write(cache_layer, pool: int, positions, token_segment, block_tables, kv_heads: int, dk: int, dv: int,
-                  page_size: int):
+def kv_pool_write(cache_layer, pooled, pool: int, positions, token_segment, block_tables, pool_tables, kv_heads: int, dk: int,
+                  dv: int, page_size: int):
     """Behind the launch that wrote a step's keys and values: every token at the last position of a block of
-    `pool` positions leaves the means of the block's keys and values, as the cache holds them, in the pages'
-    second section under the block's number."""
-    _gpu(cache_layer, positions, token_segment, block_tables)
+    `pool` positions leaves the means of the block's keys and values, as `cache_layer` holds them, in entry
+    (position // pool) of the cache layer `pooled` (the tokens' page shape, block tables `pool_tables`)."""
+    _gpu(cache_layer, pooled, positions, token_segment, block_tables, pool_tables)
     n = positions.numel()
     _check(pool >= 1, "kv_pool_write: a block holds at least one position")
-    _kv_cache(cache_layer, kv_heads, dk, dv, page_size, "kv_pool_write", 2)
+    _kv_cache(cache_layer, kv_heads, dk, dv, page_size, "kv_pool_write")
     _i32(positions, "kv_pool_write positions", n)
     _i32(token_segment, "kv_pool_write token_segment", n)
     _check(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.stride(1) == 1,
            "kv_pool_write: block tables")
-    lib.core().call("hfee_kv_pool_write", _ptr(cache_layer), _dt(cache_layer), int(pool), _ptr(positions), _ptr(token_segment),
-                    _ptr(block_tables), block_tables.stride(0), kv_heads, dk, dv, page_size, n, _stream())
+    pooled, pool_tables, pool_stride = _sight(1, pool, 0.0, pooled, pool_tables, cache_layer, block_tables.shape[0], "kv_pool_write")
+    lib.core().call("hfee_kv_pool_write", _ptr(cache_layer), _ptr(pooled), _dt(cache_layer), int(pool), _ptr(positions),
+                    _ptr(token_segment), _ptr(block_tables), block_tables.stride(0), _ptr(pool_tables), pool_stride, kv_heads, dk,
+                    dv, page_size, n, _stream())
 
 
 def qk_norm_write(q, k, v, positions, token_segment, block_tables, cache_layer, q_weight, k_weight, eps: float,
@@ -988,20 +1002,21 @@ def attention_kv_partial_words(num_items: int, num_heads: int, dv: int, splits: 
 
 def attention_kv_bf16(out, q, cache_layer, items, mode: int, block_tables, num_heads: int, kv_heads: int, dk: int,
                       dv: int, page_size: int, scale: float, sinks=None, partial=None, splits: int = 1,
-                      weights: str = "softmax", window: int = 0, pool: int = 0, softcap: float = 0.0, sections: int = 1,
-                      gate=None):
+                      weights: str = "softmax", window: int = 0, pool: int = 0, softcap: float = 0.0, pooled=None,
+                      pool_tables=None, gate=None):
     """Matrix-core attention, bfloat16 (weights: as in `attention_kv_plain`).  items: int32 [count, 4] on the device (first row, rows,
     first position, block-table row).  mode 0: an item is up to `attention_kv_rows` consecutive tokens of a portion;
     mode 1: an item is a single token (rows = 1), whose keys may be split over `splits` waves that
     leave partial results in `partial` (float32, `attention_kv_partial_words`) for a joining kernel.
-    window, pool, softcap, sections, gate: as in `attention_kv_plain`."""
-    _gpu(out, q, cache_layer, items, block_tables, sinks, partial, gate)
-    _sight(window, pool, softcap, sections, "attention_kv")
+    window, pool, softcap, pooled, pool_tables, gate: as in `attention_kv_plain`."""
+    _gpu(out, q, cache_layer, items, block_tables, sinks, partial, gate, pooled, pool_tables)
     n, w, ldq = _rows2d(q, "attention_kv q")
     no, wo, ldo = _rows2d(out, "attention_kv out")
     _check(no == n and w == num_heads * dk and wo == num_heads * dv, "attention_kv: q/out shape")
     _check(q.dtype == out.dtype == cache_layer.dtype == torch.bfloat16, "attention_kv: bfloat16 tensors expected")
-    _kv_cache(cache_layer, kv_heads, dk, dv, page_size, "attention_kv", sections)
+    _kv_cache(cache_layer, kv_heads, dk, dv, page_size, "attention_kv")
+    pooled, pool_tables, pool_stride = _sight(window, pool, softcap, pooled, pool_tables, cache_layer, block_tables.shape[0],
+                                              "attention_kv")
     ldg = 0
     if gate is not None:
         ng, wg, ldg = _rows2d(gate, "attention_kv gate")
@@ -1019,7 +1034,7 @@ def attention_kv_bf16(out, q, cache_layer, items, mode: int, block_tables, num_h
         "hfee_attention_kv_bf16", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), _ptr(items), items.shape[0], int(mode),
         _ptr(block_tables), block_tables.stride(0), num_heads, kv_heads, page_size, float(scale), _ptr(sinks),
         _ptr(partial), 0 if partial is None else partial.numel(), int(splits), int(window), int(pool), float(softcap),
-        int(sections), _ptr(gate), ldg, _stream())
+        _ptr(pooled), _ptr(pool_tables), pool_stride, _ptr(gate), ldg, _stream())
 
 
 def head_linear(out, x, weight, heads: int, n_in: int, n_out: int, tail: int = 0, x_head_stride: int | None = None,

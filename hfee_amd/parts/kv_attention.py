@@ -34,8 +34,8 @@ request are state); q and k are rotated; with `value_norm_eps` a head's value is
 square and cached so; score = q.k * scale, with `softcap` c then c * tanh(score / c); a query sees the last
 `window` positions and, with `pool` = P, one key and one value for every block of P positions that lies
 wholly before the window (the means of the block's cached keys and values, made when the block's last token
-is written, in the second section of the layer's pages under the block's number); tokens and blocks share
-one softmax; with `head_gate` a head's result is multiplied by sigmoid(W_g h)_h.
+is written, in a second cache layer that grows by one entry every P tokens, under the block's number); tokens
+and blocks share one softmax; with `head_gate` a head's result is multiplied by sigmoid(W_g h)_h.
 
 "sigmoid_attention": grouped attention without a softmax and without a rotation.  q and k are divided
 by their root mean square over each head (eps `norm_eps`) and multiplied by a weight of the head's size
@@ -85,7 +85,7 @@ def plan_items(plan, rows: int) -> None:
 def attend(ctx, out, q, cache, tables, num_heads, kv_heads, dk, dv, scale, sinks, matrix: bool, weights: str = "softmax",
            sight=None, gate=None) -> None:
     """weights "sigmoid": no softmax, `sinks` holds the number a head that joins every score.  sight: None, or
-    dict(window, pool, softcap, sections) of a mixer whose queries do not see every earlier key as it is."""
+    dict(window, pool, softcap, pooled, pool_tables) of a mixer whose queries do not see every earlier key as it is."""
     sight = sight or {}
     if not matrix:
         ops.attention_kv_plain(out, q, cache, ctx.positions, ctx.token_segment, tables, num_heads, kv_heads, dk, dv,
@@ -461,10 +461,8 @@ class WindowAttention(_KvMixer):
         self.q_width, self.k_width, self.v_width = self.num_heads * self.dk, self.kv_heads * self.dk, self.kv_heads * self.dv
         self.out_width = self.num_heads * self.dv
         self.channels = self.q_width + self.k_width + self.v_width
-        self.sections = 2 if self.pool else 1
         self.kernel_sizes = (self.dk, self.dv, self.num_heads // self.kv_heads)
         self.matrix = self._matrix(self.dk, self.dv, self.q_width, self.out_width)
-        self.sight = dict(window=self.window, pool=self.pool, softcap=self.softcap, sections=self.sections)
 
     def tensor_specs(self):
         n = self.names
@@ -492,11 +490,18 @@ class WindowAttention(_KvMixer):
         self.w_in_tiles, self.w_o_tiles = tiles_of(self.dtype, self.w_in, self.w_o)
 
     def cache_spec(self):
-        return CacheNeed("full", (self.kv_heads, self.sections, self.dk + self.dv), 0, layout=_LAYOUT)
+        # a token is read by the queries of the next `window` positions and, once more, when its block is pooled
+        keep = max(self.window, self.pool)
+        tokens = CacheNeed("window" if self.window else "full", (self.kv_heads, self.dk + self.dv), keep if self.window else 0,
+                           layout=_LAYOUT)
+        if not self.pool:
+            return tokens
+        # the pooled blocks: a second cache layer, one entry of the tokens' shape every `pool` tokens
+        return (tokens, CacheNeed("full", (self.kv_heads, self.dk + self.dv), 0, layout=_LAYOUT, every=self.pool))
 
     def key_layout(self):
         pos = self.position
-        return (self.kv_heads, self.dk, self.dv, self.sections, self.pool, self.taps, self.value_norm_eps,
+        return (self.kv_heads, self.dk, self.dv, self.pool, self.taps, self.value_norm_eps,
                 None if pos is None else pos.signature())
 
     def state_specs(self):
@@ -511,8 +516,12 @@ class WindowAttention(_KvMixer):
             raise ValueError("window_attention keeps its own keys: a request's convolution state belongs to one run of the layer")
         hn = h.tensor() if isinstance(h, LazyNorm) else h
         H, G, dk, dv = self.num_heads, self.kv_heads, self.dk, self.dv
-        cache = ctx.storage.layer(cache_layer, (G, self.sections * ctx.page_size * (dk + dv)))
+        cache = ctx.storage.layer(cache_layer, (G, ctx.page_size * (dk + dv)))
         tables = self._tables(ctx, cache_layer)
+        sight = dict(window=self.window, pool=self.pool, softcap=self.softcap)
+        if self.pool:
+            sight.update(pooled=ctx.storage.layer((cache_layer, 1), (G, ctx.page_size * (dk + dv))),
+                         pool_tables=self._tables(ctx, (cache_layer, 1)))
         pos = self.position
         cos, sin = (pos.cos, pos.sin) if pos else (None, None)
         total = self.w_in.shape[0]       # (rows of a multiple of 8 elements, so that blocks of columns stay aligned)
@@ -529,11 +538,11 @@ class WindowAttention(_KvMixer):
         q = ctx.rows("window_attention.q", self.q_width)
         ops.rotate_norm_write(q, qkv[:, :self.q_width], qkv[:, self.q_width:self.q_width + self.k_width],
                               qkv[:, self.q_width + self.k_width:], ctx.positions, ctx.token_segment, tables, cos, sin, cache,
-                              H, G, dk, dv, ctx.page_size, ctx.max_position, value_eps=self.value_norm_eps,
-                              sections=self.sections)
+                              H, G, dk, dv, ctx.page_size, ctx.max_position, value_eps=self.value_norm_eps)
         if self.pool:
-            ops.kv_pool_write(cache, self.pool, ctx.positions, ctx.token_segment, tables, G, dk, dv, ctx.page_size)
+            ops.kv_pool_write(cache, sight["pooled"], self.pool, ctx.positions, ctx.token_segment, tables, sight["pool_tables"],
+                              G, dk, dv, ctx.page_size)
         gate = proj[:, self.channels:self.channels + H] if self.has_gate else None
         att = ctx.rows("kv_attention.out", self.out_width)
-        attend(ctx, att, q, cache, tables, H, G, dk, dv, self.scale, None, self.matrix, sight=self.sight, gate=gate)
+        attend(ctx, att, q, cache, tables, H, G, dk, dv, self.scale, None, self.matrix, sight=sight, gate=gate)
         product(ctx, out, att, self.w_o, self.w_o_tiles)

@@ -76,6 +76,39 @@ def test_window_group_gives_back_pages_the_window_has_passed():
     assert m.free_pages() == [32, 12]
 
 
+def test_a_group_that_grows_every_few_tokens():
+    """One entry every 5 tokens: n tokens hold ceil(n / 5) entries in ceil(ceil(n / 5) / 16) pages; a
+    reservation fails as a whole when that group alone has no page left; truncation cuts it back too."""
+    every5 = CacheGroupSpec("full", (2, 24), cache_layers=((0, 1),), every=5)
+    m = CacheManager([FULL, every5], 16, [40, 3], max_requests=2)
+    m.admit("r")
+    n = 0
+    for portion in (1, 3, 1, 75, 1, 79, 1, 2, 77):
+        m.reserve("r", portion)
+        m.commit("r", portion)
+        n += portion
+        m.check()
+        entries = (n + 4) // 5
+        assert len(m.block_table("r", 0)) == (n + 15) // 16 and len(m.block_table("r", 1)) == (entries + 15) // 16
+    assert n == 240 and m.pages_needed("r", 1) == [1, 1] and m.pages_for_tokens(161) == [11, 3]
+    m.admit("s")
+    with pytest.raises(OutOfPages):
+        m.reserve("s", 1)                  # (the tokens' group has pages, the other has none)
+    assert m.block_table("s", 0) == [] and m.free_pages() == [25, 0]
+    m.truncate("r", 80)
+    assert len(m.block_table("r", 0)) == 5 and len(m.block_table("r", 1)) == 1 and m.free_pages() == [35, 2]
+    m.reserve("s", 81)
+    m.commit("s", 81)
+    m.check()
+    m.release("r")
+    m.release("s")
+    assert m.free_pages() == [40, 3]
+    with pytest.raises(CacheError):
+        CacheGroupSpec("window", (2, 24), cache_layers=(3,), window=8, every=2)
+    with pytest.raises(CacheError):
+        CacheManager([FULL, every5], 16, [8, 8], max_requests=1, keep_prefixes=True)
+
+
 @pytest.mark.parametrize("seed", range(8))
 def test_random_orders_keep_every_invariant(seed):
     rng = random.Random(seed)

@@ -108,13 +108,18 @@ def test_attention_over_a_window_with_pooled_blocks(dtype, H, G, dk, dv, window,
             ks[0][j, kv1] = qs[0][last - n_back % 3, 1] * 3.0
     qs, ks, vs = ([t.to(dt).float() for t in x] for x in (qs, ks, vs))
     gates = [None if t is None else t.to(dt).float() for t in gates]
-    sections = 2 if pool and window else 1
+    pooling = bool(pool and window)
     tables, pages = _paged(lengths)
-    cache = torch.zeros(pages, G, sections * 16 * (dk + dv), dtype=dt, device="cuda")
+    cache = torch.zeros(pages, G, 16 * (dk + dv), dtype=dt, device="cuda")
     cache[0].fill_(float("nan"))
     bt = i32(tables)
     matrix = dtype == "bfloat16" and ops.attention_kv_sizes_fit(dk, dv)
-    sight = dict(window=window, pool=pool if window else 0, softcap=cap, sections=sections)
+    sight = dict(window=window, pool=pool if window else 0, softcap=cap)
+    if pooling:        # the pooled blocks: a cache layer of their own that grows by an entry every `pool` tokens
+        pool_tables, pool_pages = _paged([-(-n // pool) for n in lengths], seed=1)
+        pooled = torch.zeros(pool_pages, G, 16 * (dk + dv), dtype=dt, device="cuda")
+        pooled[0].fill_(float("nan"))
+        pbt = i32(pool_tables)
     # the values as the cache holds them: normed a head, rounded
     eps = 1e-5
     vn = [(v.double() / torch.sqrt((v.double() ** 2).mean(-1, keepdim=True) + eps)).to(dt).double() for v in vs]
@@ -132,9 +137,10 @@ def test_attention_over_a_window_with_pooled_blocks(dtype, H, G, dk, dv, window,
         tab = bt[[s for s, _ in segs]].contiguous()
         q = torch.zeros(n_all, H * dk, dtype=dt, device="cuda")
         ops.rotate_norm_write(q, q32, k32, v32, positions, token_segment, tab, None, None, cache, H, G, dk, dv, 16,
-                              int(positions.max()), value_eps=eps, sections=sections)
-        if sections == 2:
-            ops.kv_pool_write(cache, pool, positions, token_segment, tab, G, dk, dv, 16)
+                              int(positions.max()), value_eps=eps)
+        if pooling:
+            sight.update(pooled=pooled, pool_tables=pbt[[s for s, _ in segs]].contiguous())
+            ops.kv_pool_write(cache, pooled, pool, positions, token_segment, tab, sight["pool_tables"], G, dk, dv, 16)
         out = torch.zeros(n_all, H * dv, dtype=dt, device="cuda")
         ops.attention_kv_plain(out, q, cache, positions, token_segment, tab, H, G, dk, dv, 16, scale, gate=gate, **sight)
         outs = [out]
@@ -170,7 +176,7 @@ def test_attention_over_a_window_with_pooled_blocks(dtype, H, G, dk, dv, window,
             fed[s] += n
             row += n
     assert fed == lengths
-    assert torch.isnan(cache[0].float()).all()
+    assert torch.isnan(cache[0].float()).all() and (not pooling or torch.isnan(pooled[0].float()).all())
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -188,23 +194,22 @@ def test_rotation_and_value_norm_on_the_way_into_the_cache(dtype):
     table_sin = torch.zeros(start + n, rot // 2, device="cuda")
     table_cos[start:], table_sin[start:] = cos, sin
     tables, pages = _paged([start + n])
-    for sections in (1, 2):
-        cache = torch.zeros(pages, G, sections * 16 * (dk + dv), dtype=dt, device="cuda")
-        q_out = torch.zeros(n, H * dk, dtype=dt, device="cuda")
-        ops.rotate_norm_write(q_out, q.cuda(), k.cuda(), v.cuda(), i32(pos), i32(np.zeros(n)), i32(tables), table_cos, table_sin,
-                              cache, H, G, dk, dv, 16, start + n - 1, value_eps=1e-3, sections=sections)
-        want_q = ps.rotate_half(q.double().view(n, H, dk), pos, rot, 300.0).reshape(n, -1)
-        want_k = ps.rotate_half(k.double().view(n, G, dk), pos, rot, 300.0)
-        want_v = ps.rms(v.double().view(n, G, dv), 1e-3)
-        tol = 1e-6 if dtype == "float32" else 1e-2
-        assert su.rel(q_out.double().cpu(), want_q) < tol
-        pages_of = cache.view(pages, G, sections, 16 * (dk + dv)).double().cpu()
-        for t in range(n):
-            p = start + t
-            page, slot = tables[0, p // 16], p % 16
-            keys = pages_of[page, :, 0, :16 * dk].view(G, 16, dk)[:, slot]
-            values = pages_of[page, :, 0, 16 * dk:].view(G, dv, 16)[:, :, slot]
-            assert su.rel(keys, want_k[t]) < tol and su.rel(values, want_v[t]) < tol
+    cache = torch.zeros(pages, G, 16 * (dk + dv), dtype=dt, device="cuda")
+    q_out = torch.zeros(n, H * dk, dtype=dt, device="cuda")
+    ops.rotate_norm_write(q_out, q.cuda(), k.cuda(), v.cuda(), i32(pos), i32(np.zeros(n)), i32(tables), table_cos, table_sin,
+                          cache, H, G, dk, dv, 16, start + n - 1, value_eps=1e-3)
+    want_q = ps.rotate_half(q.double().view(n, H, dk), pos, rot, 300.0).reshape(n, -1)
+    want_k = ps.rotate_half(k.double().view(n, G, dk), pos, rot, 300.0)
+    want_v = ps.rms(v.double().view(n, G, dv), 1e-3)
+    tol = 1e-6 if dtype == "float32" else 1e-2
+    assert su.rel(q_out.double().cpu(), want_q) < tol
+    pages_of = cache.double().cpu()
+    for t in range(n):
+        p = start + t
+        page, slot = tables[0, p // 16], p % 16
+        keys = pages_of[page, :, :16 * dk].view(G, 16, dk)[:, slot]
+        values = pages_of[page, :, 16 * dk:].view(G, dv, 16)[:, :, slot]
+        assert su.rel(keys, want_k[t]) < tol and su.rel(values, want_v[t]) < tol
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -431,6 +436,23 @@ def test_a_slot_that_is_used_again_starts_from_nothing(folders, plain_rows, name
     rep = Replayer(folders[(name, "float32")], "float32", (longest + 63) // 64 * 64, max_requests=1)
     got = tu.run(rep, tu.portions(reqs, sizes=(9, 2, 30)))
     compare(got, want, "float32", f"{name}: one slot for all")
+
+
+def test_the_pooled_blocks_take_a_page_every_so_many_tokens(folders, plain_rows):
+    """The attention layer's pooled blocks are a cache group that grows by an entry every `pool` tokens: a request
+    of 150 tokens with blocks of 3 holds 50 entries of it, four pages; its tokens are a window group that keeps the
+    window's pages only."""
+    from hfee_amd.trace_replay import Replayer
+    reqs, want = plain_rows("attention", "float32", [150])
+    rep = Replayer(folders[("attention", "float32")], "float32", 192, max_requests=2)
+    groups = rep.engine.cache.groups
+    assert sorted((g.every, g.kind, g.window, g.cache_layers) for g in groups) == [(1, "window", 10, (0,)), (3, "full", 0, ((0, 1),))]
+    rows = rep.step([("r0", reqs["r0"], list(range(150)))])
+    held = {groups[g].every: sum(p >= 0 for p in t) for g, t in enumerate(rep.engine.cache.get("r0").tables)}
+    assert held == {1: 2, 3: 4}            # (the next query reads the positions from 141 on: the ninth and tenth page)
+    compare({("r0", i): rows[i] for i in range(150)}, want, "float32", "a group that grows every third token")
+    rep.engine.release("r0")
+    rep.engine.cache.check()
 
 
 def test_a_window_gives_back_the_pages_it_has_passed(folders, plain_rows):

@@ -96,6 +96,27 @@ def make(num_pages=64, seqs=4, budget=32, ctx=256, eos=(), keep_prefixes=False):
                           eos_token_ids=eos, clock=lambda: 0.0)
 
 
+def test_a_group_that_grows_every_few_tokens_holds_that_many_tokens_a_page():
+    """Beside the tokens' group a group with an entry every 8 tokens and three pages: they hold 384 tokens' worth,
+    so three requests of 100 tokens each run side by side without anybody giving way, as the same requests do
+    with that group as large as the tokens'; with two pages the youngest has to wait, and all three still end
+    with the same tokens."""
+    def run(pages):
+        eng = FakeEngine(64, 4)
+        groups = [CacheGroupSpec("full", (2, 1, 16), (0,)), CacheGroupSpec("full", (2, 1, 16), ((0, 1),), every=8)]
+        eng.cache = CacheManager(groups, 16, [64, pages], 4)
+        s = Scheduler(eng, FakeSampler(), max_num_seqs=4, max_batch_tokens=64, num_ctx=256, clock=lambda: 0.0)
+        for i in range(3):
+            s.add(Request(i, [(5 * i + j) % (VOCAB - 1) for j in range(70)], SamplingParams.greedy(num_predict=30), seed=i))
+        done = run_all(s)
+        eng.cache.check()
+        assert eng.cache.free_pages() == [64, pages]
+        return {i: (f.request.generated, f.request.stats.done_reason, f.request.stats.preemptions) for i, f in done.items()}
+    roomy, enough, scarce = run(64), run(3), run(2)
+    assert roomy == enough and all(reason == "length" and pre == 0 and len(g) == 30 for g, reason, pre in enough.values())
+    assert {i: g for i, (g, _, _) in scarce.items()} == {i: g for i, (g, _, _) in roomy.items()}
+
+
 def run_all(sched, limit=10000):
     done = {}
     for _ in range(limit):
