@@ -249,7 +249,6 @@ class Scheduler:
         self._preempted_now.clear()
 
         # decoding requests first, oldest first; preempt from the young end if pages run out
-        ps = self.cache.page_size
         for r in [x for x in self.running if x.decoding]:
             if r not in self.running:
                 continue          # preempted while an older request was served

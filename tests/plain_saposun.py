@@ -8,8 +8,6 @@ walks over it token by token, so cutting a sequence can change nothing here.
 """
 from __future__ import annotations
 
-import math
-
 import torch
 import torch.nn.functional as F
 

@@ -16,7 +16,6 @@ import sys
 import numpy as np
 import pytest
 import torch
-import torch.nn.functional as F
 
 import plain_saposun as ps
 import saposun_util as su
